@@ -1,0 +1,85 @@
+// Host-only part of the C ABI: version, error reporting, argument validation.
+#include <cstdarg>
+#include <cstdio>
+
+#include "tf24_common.hpp"
+
+namespace tf24 {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof g_error, fmt, ap);
+  va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof g_error, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TF24_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return TF24_OK;
+}
+
+static bool is_float_dtype(int dt) { return dt == TF24_F32 || dt == TF24_F16 || dt == TF24_BF16; }
+static bool is_mask_dtype(int dt) { return dt == TF24_U8 || is_float_dtype(dt); }
+static bool is_layout(int l) { return l == TF24_ROW_MAJOR || l == TF24_COL_MAJOR; }
+
+// leading dimension of an [m,k] matrix: at least the contiguous extent, and a multiple of 8
+// elements so that every 128-bit access stays aligned
+static int check_ld(const char* fn, const char* name, int layout, int64_t ld, int64_t m, int64_t k) {
+  int64_t extent = layout == TF24_ROW_MAJOR ? k : m;
+  if (ld < extent) return fail(TF24_ERR_STRIDE, "%s: %s leading dimension %lld < %lld", fn, name, (long long)ld, (long long)extent);
+  if (ld % 8) return fail(TF24_ERR_STRIDE, "%s: %s leading dimension %lld must be a multiple of 8", fn, name, (long long)ld);
+  return TF24_OK;
+}
+
+}  // namespace tf24
+
+using namespace tf24;
+
+extern "C" const char* tf24_version(void) { return "tf24 0.1.0 gfx950"; }
+
+extern "C" const char* tf24_last_error(void) { return g_error; }
+
+extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld, int64_t m, int64_t k, int mode,
+                                            int has_mask, int mask_dtype, int64_t mask_ld, int has_rand, int64_t rand_ld,
+                                            int out_dtype) {
+  const char* fn = "tf24_prune_compress";
+  if (!is_float_dtype(in_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
+  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && out_dtype != TF24_E4M3)
+    return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
+  if (!is_layout(layout)) return fail(TF24_ERR_ARG, "%s: bad layout %d", fn, layout);
+  const int64_t min_rows = 32, min_cols = out_dtype == TF24_E4M3 ? 128 : 64;
+  if (m < min_rows || m % min_rows || k < min_cols || k % min_cols)
+    return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld) is not supported: both dimensions must be >= and a multiple of (%lld, %lld)",
+                fn, (long long)m, (long long)k, (long long)min_rows, (long long)min_cols);
+  if (m * (k / 8) > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "%s: matrix too large (%lld x %lld)", fn, (long long)m, (long long)k);
+  int rc = check_ld(fn, "dense", layout, ld, m, k);
+  if (rc) return rc;
+  switch (mode) {
+    case TF24_PRUNE_MAGNITUDE:
+      break;
+    case TF24_PRUNE_MASK:
+      if (!has_mask) return fail(TF24_ERR_ARG, "%s: mode MASK needs a mask", fn);
+      if (!is_mask_dtype(mask_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported mask dtype %d", fn, mask_dtype);
+      if ((rc = check_ld(fn, "mask", layout, mask_ld, m, k))) return rc;
+      break;
+    case TF24_PRUNE_MVUE:
+      if (!has_rand) return fail(TF24_ERR_ARG, "%s: mode MVUE needs a rand tensor", fn);
+      if ((rc = check_ld(fn, "rand", layout, rand_ld, m, k))) return rc;
+      break;
+    default:
+      return fail(TF24_ERR_ARG, "%s: bad mode %d", fn, mode);
+  }
+  if (has_mask && has_rand) return fail(TF24_ERR_ARG, "%s: using MVUE24 with mask is not supported", fn);
+  return TF24_OK;
+}

@@ -1,0 +1,58 @@
+// Compressed 2:4 -> dense for gfx950.  Lane owns 8 dense outputs (two groups): loads its 4 kept
+// values and one metadata byte, stores 8 elements with one vector store.
+#include "tf24_common.hpp"
+
+namespace tf24 {
+namespace {
+
+constexpr int kThreads = 256;
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta, int64_t total_units, T* __restrict__ dense) {
+  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (u >= total_units) return;
+  Pack<T, 4> v;
+  v.load(values + u * 4);
+  const uint32_t mb = meta[u];
+  Pack<T, 8> out;
+#pragma unroll
+  for (int i = 0; i < 8; i++) out.v[i] = T{};
+#pragma unroll
+  for (int g = 0; g < 2; g++) {
+    const uint32_t nib = (mb >> (4 * g)) & 0xf;
+    const uint32_t p0 = nib & 3, p1 = nib >> 2;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      if (p0 == (uint32_t)i) out.v[4 * g + i] = v.v[2 * g];
+      if (p1 == (uint32_t)i) out.v[4 * g + i] = v.v[2 * g + 1];
+    }
+  }
+  out.store(dense + u * 8);
+}
+
+template <typename T>
+int launch(const void* values, const void* meta, int64_t m, int64_t k, void* dense, hipStream_t s) {
+  const int64_t total = m * (k / 8);
+  dim3 grid((unsigned)((total + kThreads - 1) / kThreads));
+  hipLaunchKernelGGL((decompress_kernel<T>), grid, dim3(kThreads), 0, s, (const T*)values, (const uint8_t*)meta, total, (T*)dense);
+  return check_launch("tf24_decompress");
+}
+
+}  // namespace
+}  // namespace tf24
+
+extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, int64_t m, int64_t k,
+                               void* dense_out, void* stream) {
+  using namespace tf24;
+  const int64_t mult = dtype == TF24_E4M3 ? 32 : 16;
+  if (m <= 0 || k <= 0 || k % mult) return fail(TF24_ERR_SHAPE, "tf24_decompress: k=%lld must be a positive multiple of %lld", (long long)k, (long long)mult);
+  if (!values || !meta || !dense_out) return fail(TF24_ERR_ARG, "tf24_decompress: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case TF24_F16: return launch<f16_t>(values, meta, m, k, dense_out, s);
+    case TF24_BF16: return launch<bf16_t>(values, meta, m, k, dense_out, s);
+    case TF24_E4M3: return launch<e4m3_t>(values, meta, m, k, dense_out, s);
+  }
+  return fail(TF24_ERR_DTYPE, "tf24_decompress: unsupported dtype %d", dtype);
+}

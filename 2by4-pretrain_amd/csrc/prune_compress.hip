@@ -1,0 +1,259 @@
+// Dense -> 2:4 prune + compress for gfx950 (HBM-bound streaming kernels).
+//
+// Row-major input: one lane owns 8 consecutive elements (two groups): 128-bit loads for 16-bit
+// inputs, 4 kept values leave as one 64-bit (16-bit values) or 32-bit (fp8) store, and the lane's
+// metadata byte is merged across 4 lanes with wave shuffles into one 32-bit store.
+// Column-major input (W.T, dY.t() views): one lane owns a 4-column x R-row sub-tile (R groups that
+// live entirely in its registers), a 256-lane block covers 8R rows x 128 columns, and the
+// compressed tile is transposed through LDS so that values and metadata leave row-major with
+// full-line stores.
+#include "tf24_common.hpp"
+
+namespace tf24 {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+template <typename In, int MODE, typename MaskT>
+__device__ __forceinline__ uint32_t prune_group(const float (&x)[4], const MaskT* mk, float r0, float r1, float (&y)[4]) {
+  if constexpr (MODE == TF24_PRUNE_MAGNITUDE) {
+    y[0] = x[0]; y[1] = x[1]; y[2] = x[2]; y[3] = x[3];
+    return magnitude_mask4(x[0], x[1], x[2], x[3]);
+  } else if constexpr (MODE == TF24_PRUNE_MASK) {
+    y[0] = x[0]; y[1] = x[1]; y[2] = x[2]; y[3] = x[3];
+    uint32_t b = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) b |= (uint32_t)(to_float(mk[i]) != 0.0f) << i;
+    return b;
+  } else {
+    return mvue4(x[0], x[1], x[2], x[3], r0, r1, y[0], y[1], y[2], y[3]);
+  }
+}
+
+// ------------------------------------------------------------------ row-major
+template <typename In, typename Out, int MODE, typename MaskT>
+__global__ void __launch_bounds__(kThreads)
+prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
+                   const MaskT* __restrict__ mask, int64_t mask_ld,
+                   const float* __restrict__ rnd, int64_t rand_ld,
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous) {
+  const int64_t upr = k >> 3;                 // 8-element units per row
+  const int64_t total = m * upr;
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+#pragma unroll
+  for (int it = 0; it < kUnroll; it++) {
+    const int64_t u = base + (int64_t)it * kThreads;
+    const bool live = u < total;
+    uint32_t mbyte = 0;
+    Pack<Out, 4> out;
+    int64_t row = 0, col8 = 0;
+    if (live) {
+      if (contiguous) {          // every leading dimension equals k: offsets are linear in u
+        col8 = u;
+      } else {
+        row = (int64_t)((uint32_t)u / (uint32_t)upr);
+        col8 = u - row * upr;
+      }
+      Pack<In, 8> in;
+      in.load(dense + row * ld + col8 * 8);
+      Pack<MaskT, 8> mk;
+      float r[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (MODE == TF24_PRUNE_MASK) mk.load(mask + row * mask_ld + col8 * 8);
+      if constexpr (MODE == TF24_PRUNE_MVUE) {
+        const float* rp = rnd + row * rand_ld + col8 * 8;
+        float2 ra = *reinterpret_cast<const float2*>(rp);
+        float2 rb = *reinterpret_cast<const float2*>(rp + 4);
+        r[0] = ra.x; r[1] = ra.y; r[2] = rb.x; r[3] = rb.y;
+      }
+#pragma unroll
+      for (int g = 0; g < 2; g++) {
+        float x[4], y[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = to_float(in.v[4 * g + i]);
+        uint32_t mb = prune_group<In, MODE, MaskT>(x, &mk.v[4 * g], r[2 * g], r[2 * g + 1], y);
+        uint32_t nib = encode_nibble(mb);
+        out.v[2 * g] = from_float<Out>(select4(nib & 3, y[0], y[1], y[2], y[3]));
+        out.v[2 * g + 1] = from_float<Out>(select4(nib >> 2, y[0], y[1], y[2], y[3]));
+        mbyte |= nib << (4 * g);
+      }
+      out.store(values + row * (k >> 1) + col8 * 4);
+    }
+    // 4 adjacent lanes (32 dense columns of one row) -> one metadata dword
+    uint32_t w = mbyte;
+    w |= __shfl_down(mbyte, 1) << 8;
+    w |= __shfl_down(mbyte, 2) << 16;
+    w |= __shfl_down(mbyte, 3) << 24;
+    if (live && (threadIdx.x & 3) == 0)
+      *reinterpret_cast<uint32_t*>(meta + row * (k >> 3) + col8) = w;
+  }
+}
+
+// ------------------------------------------------------------------ column-major
+// element (r,c) at c*ld + r.  R = rows per lane = 16 bytes / sizeof(In).
+template <typename In, typename Out, int MODE, typename MaskT>
+__global__ void __launch_bounds__(kThreads)
+prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
+                   const MaskT* __restrict__ mask, int64_t mask_ld,
+                   const float* __restrict__ rnd, int64_t rand_ld,
+                   Out* __restrict__ values, uint8_t* __restrict__ meta) {
+  constexpr int R = 16 / sizeof(In);
+  constexpr int TR = 8 * R;          // tile rows
+  constexpr int TC = 128;            // tile columns (32 groups)
+  constexpr int VPITCH = (TC / 2) * sizeof(Out) + 4;   // bytes per row of the value tile (+1 bank)
+  constexpr int MPITCH = TC / 8 + 4;                   // bytes per row of the metadata tile
+  __shared__ __attribute__((aligned(16))) uint8_t s_val[TR * VPITCH];
+  __shared__ __attribute__((aligned(16))) uint8_t s_meta[TR * MPITCH];
+
+  const int tid = threadIdx.x;
+  const int rchunk = tid & 7, grp = tid >> 3;           // 8 row chunks x 32 groups
+  const int64_t row0 = (int64_t)blockIdx.y * TR, col0 = (int64_t)blockIdx.x * TC;
+  const int64_t r0 = row0 + rchunk * R, c0 = col0 + grp * 4;
+  if (r0 < m && c0 < k) {
+    Pack<In, R> in[4];
+    Pack<MaskT, R> mk[4];
+    Pack<float, R> rr[2];
+#pragma unroll
+    for (int c = 0; c < 4; c++) in[c].load(dense + (c0 + c) * ld + r0);
+    if constexpr (MODE == TF24_PRUNE_MASK) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) mk[c].load(mask + (c0 + c) * mask_ld + r0);
+    }
+    if constexpr (MODE == TF24_PRUNE_MVUE) {
+      rr[0].load(rnd + (c0 + 0) * rand_ld + r0);
+      rr[1].load(rnd + (c0 + 1) * rand_ld + r0);
+    }
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+      float x[4], y[4];
+      MaskT mrow[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) { x[c] = to_float(in[c].v[i]); if constexpr (MODE == TF24_PRUNE_MASK) mrow[c] = mk[c].v[i]; }
+      float u0 = 0.f, u1 = 0.f;
+      if constexpr (MODE == TF24_PRUNE_MVUE) { u0 = rr[0].v[i]; u1 = rr[1].v[i]; }
+      uint32_t mb = prune_group<In, MODE, MaskT>(x, mrow, u0, u1, y);
+      uint32_t nib = encode_nibble(mb);
+      Pack<Out, 2> o;
+      o.v[0] = from_float<Out>(select4(nib & 3, y[0], y[1], y[2], y[3]));
+      o.v[1] = from_float<Out>(select4(nib >> 2, y[0], y[1], y[2], y[3]));
+      const int lr = rchunk * R + i;
+      o.store(reinterpret_cast<Out*>(s_val + lr * VPITCH) + grp * 2);
+      // two groups share a metadata byte: even group low nibble, odd group high nibble
+      uint32_t other = __shfl_xor(nib, 8);     // lane with grp^1 (same rchunk)
+      if ((grp & 1) == 0) s_meta[lr * MPITCH + (grp >> 1)] = (uint8_t)(nib | (other << 4));
+    }
+  }
+  __syncthreads();
+  // values: TR rows x (TC/2)*sizeof(Out) bytes, 16 bytes per lane
+  constexpr int VROW_BYTES = (TC / 2) * sizeof(Out);
+  constexpr int LANES_PER_ROW = VROW_BYTES / 16;
+  constexpr int ROWS_PER_PASS = kThreads / LANES_PER_ROW;
+  const int64_t vpitch_out = (k >> 1) * sizeof(Out);
+#pragma unroll
+  for (int pass = 0; pass < (TR + ROWS_PER_PASS - 1) / ROWS_PER_PASS; pass++) {
+    const int lr = pass * ROWS_PER_PASS + tid / LANES_PER_ROW;
+    const int seg = tid % LANES_PER_ROW;
+    const int64_t gr = row0 + lr;
+    const int64_t gbyte = (col0 >> 1) * sizeof(Out) + seg * 16;
+    if (lr < TR && gr < m && gbyte < vpitch_out) {
+      // LDS rows are padded by 4 bytes, so read as four dwords
+      const uint32_t* sp = reinterpret_cast<const uint32_t*>(s_val + lr * VPITCH + seg * 16);
+      uint4 v = make_uint4(sp[0], sp[1], sp[2], sp[3]);
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(values) + gr * vpitch_out + gbyte) = v;
+    }
+  }
+  // metadata: TR rows x 16 bytes
+  if (tid < TR) {
+    const int64_t gr = row0 + tid;
+    if (gr < m) {
+      const uint32_t* sp = reinterpret_cast<const uint32_t*>(s_meta + tid * MPITCH);
+      const int64_t mpitch_out = k >> 3;
+      uint8_t* dst = meta + gr * mpitch_out + (col0 >> 3);
+      // rows of the metadata matrix are only 8-byte aligned when k % 128 == 64
+      *reinterpret_cast<uint2*>(dst) = make_uint2(sp[0], sp[1]);
+      if (col0 + TC <= k) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(sp[2], sp[3]);
+    }
+  }
+}
+
+template <typename In, typename Out, int MODE, typename MaskT>
+int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
+           const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t stream) {
+  if (layout == TF24_ROW_MAJOR) {
+    const int64_t total = m * (k >> 3);
+    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == k);
+    const int64_t per_block = kThreads * kUnroll;
+    dim3 grid((unsigned)((total + per_block - 1) / per_block));
+    hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta,
+                       contiguous);
+  } else {
+    constexpr int R = 16 / sizeof(In);
+    dim3 grid((unsigned)((k + 127) / 128), (unsigned)((m + 8 * R - 1) / (8 * R)));
+    hipLaunchKernelGGL((prune_compress_col<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta);
+  }
+  return check_launch("tf24_prune_compress");
+}
+
+template <typename In, typename Out, int MODE>
+int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int mask_dtype,
+                  int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t s) {
+  if constexpr (MODE != TF24_PRUNE_MASK) {
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, values, meta, s);
+  } else {
+    switch (mask_dtype) {
+      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
+      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
+      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
+      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
+    }
+    return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported mask dtype %d", mask_dtype);
+  }
+}
+
+template <typename In, typename Out>
+int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
+                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t s) {
+  switch (mode) {
+    case TF24_PRUNE_MAGNITUDE:
+      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_PRUNE_MASK:
+      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_PRUNE_MVUE:
+      return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+  }
+  return fail(TF24_ERR_ARG, "tf24_prune_compress: bad mode %d", mode);
+}
+
+template <typename In>
+int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
+                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t s) {
+  switch (out_dtype) {
+    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+  }
+  return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported output dtype %d", out_dtype);
+}
+
+}  // namespace
+}  // namespace tf24
+
+extern "C" int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                                   int mode, const void* mask, int mask_dtype, int64_t mask_ld,
+                                   const float* rnd, int64_t rand_ld,
+                                   void* values, int out_dtype, void* meta, void* stream) {
+  using namespace tf24;
+  int rc = tf24_prune_compress_validate(in_dtype, layout, ld, m, k, mode, mask != nullptr, mask_dtype, mask_ld,
+                                        rnd != nullptr, rand_ld, out_dtype);
+  if (rc != TF24_OK) return rc;
+  if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "tf24_prune_compress: null dense/values/meta pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (in_dtype) {
+    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+  }
+  return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported input dtype %d", in_dtype);
+}

@@ -1,0 +1,212 @@
+// 2:4 sparse x dense matmul on the gfx950 sparse matrix cores (V_SMFMAC), float32 accumulation.
+//
+//     C[i,j] = act( scale * sum_k A[i,k] * B(k,j) + bias[i] )
+//
+// A is the compressed operand (values [n_sparse, k/2] + canonical metadata), which is exactly the
+// SMFMAC "A" operand: one lane holds a run of consecutive compressed values of one row and the
+// matching run of 2-bit positions is a contiguous slice of the row's metadata stream.
+//
+// Operand layouts of the instructions used (R = 16 or 32 rows, lane l, nkb = 64/R lane blocks,
+// K dense depth of the instruction, kper = K/nkb):
+//   A: row l%R, block ka = l/R holds the kper/2 compressed values of dense k in [ka*kper, (ka+1)*kper);
+//      value e uses index bits [2e+1:2e] (16-bit types: the 16-bit half of the index register
+//      selected by ABID; 8-bit types: all 32 bits)
+//   B: column l%R, block kb = l/R holds dense k in [kb*kper/2, (kb+1)*kper/2) followed by the same
+//      range shifted by K/2
+//   D: 16x16: column l%16, rows 4*(l/16)+r;  32x32: column l%32, rows 8*(r/4) + 4*(l/32) + r%4
+#include "tf24_common.hpp"
+
+namespace tf24 {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x16 __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int8v __attribute__((ext_vector_type(8)));
+
+// ---- element traits: KSTEP = dense depth of one 16x16 instruction; all types move 64 bytes of
+// compressed A and 128 bytes of B per row per step.
+template <typename T> struct mma16;
+template <> struct mma16<f16_t> {
+  static constexpr int KSTEP = 64;
+  template <int ABID>
+  static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
+    return __builtin_amdgcn_smfmac_f32_16x16x64_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half16, b), c, idx, 0, ABID);
+  }
+};
+template <> struct mma16<bf16_t> {
+  static constexpr int KSTEP = 64;
+  template <int ABID>
+  static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
+    return __builtin_amdgcn_smfmac_f32_16x16x64_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x16, b), c, idx, 0, ABID);
+  }
+};
+template <> struct mma16<e4m3_t> {
+  static constexpr int KSTEP = 128;
+  template <int ABID>
+  static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
+    return __builtin_amdgcn_smfmac_f32_16x16x128_fp8_fp8(a, b, c, idx, 0, 0);
+  }
+};
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+  if (act == TF24_ACT_RELU) return v > 0.0f ? v : 0.0f;
+  if (act == TF24_ACT_SILU) return v / (1.0f + __expf(-v));
+  return v;
+}
+
+// ------------------------------------------------------------------------------------------
+// General kernel: operands straight from global memory (cached), every supported shape and
+// layout.  One wave computes a 32(i) x 32(j) tile with 16x16 instructions; a block is 2x2 waves.
+// ------------------------------------------------------------------------------------------
+template <typename T, typename OutT, bool B_KCONTIG, bool C_JMAJOR>
+__global__ void __launch_bounds__(256)
+spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
+             const T* __restrict__ b, int64_t ldb, int64_t n_dense,
+             OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
+  constexpr int KSTEP = mma16<T>::KSTEP;
+  constexpr int ES = sizeof(T);                       // element size of values and B
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t i0 = (int64_t)blockIdx.y * 64 + (wave >> 1) * 32;
+  const int64_t j0 = (int64_t)blockIdx.x * 64 + (wave & 1) * 32;
+  if (i0 >= n_sparse || j0 >= n_dense) return;       // whole wave out of range
+  const int li = lane & 15, lk = lane >> 4;
+  const int64_t a_pitch = (k / 2) * ES;               // bytes per row of compressed values
+  const int64_t m_pitch = k / 8;                      // bytes per row of metadata
+  float4v acc[2][2];
+#pragma unroll
+  for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+    for (int tj = 0; tj < 2; tj++) acc[ti][tj] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  for (int64_t k0 = 0; k0 < k; k0 += KSTEP) {
+    int4v af[2];
+    int idx[2];
+#pragma unroll
+    for (int ti = 0; ti < 2; ti++) {
+      const int64_t row = i0 + ti * 16 + li;
+      af[ti] = *reinterpret_cast<const int4v*>(a_values + row * a_pitch + (k0 / 2) * ES + lk * 16);
+      if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(a_meta + row * m_pitch + k0 / 8 + lk * 2);
+      else idx[ti] = *reinterpret_cast<const int*>(a_meta + row * m_pitch + k0 / 8 + lk * 4);
+    }
+    int8v bf[2];
+#pragma unroll
+    for (int tj = 0; tj < 2; tj++) {
+      int64_t col = j0 + tj * 16 + li;
+      if (col >= n_dense) col = n_dense - 1;          // clamp: the column is never stored
+      constexpr int HALF = KSTEP / 8;                 // elements per half run (16 bytes)
+      if constexpr (B_KCONTIG) {
+        const T* p = b + col * ldb + k0 + lk * HALF;
+        int4v lo = *reinterpret_cast<const int4v*>(p);
+        int4v hi = *reinterpret_cast<const int4v*>(p + KSTEP / 2);
+        bf[tj] = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      } else {
+        alignas(32) T tmp[2 * HALF];
+#pragma unroll
+        for (int e = 0; e < HALF; e++) {
+          tmp[e] = b[(k0 + lk * HALF + e) * ldb + col];
+          tmp[HALF + e] = b[(k0 + KSTEP / 2 + lk * HALF + e) * ldb + col];
+        }
+        bf[tj] = *reinterpret_cast<int8v*>(tmp);
+      }
+    }
+#pragma unroll
+    for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+      for (int tj = 0; tj < 2; tj++) acc[ti][tj] = mma16<T>::template run<0>(af[ti], bf[tj], acc[ti][tj], idx[ti]);
+  }
+
+#pragma unroll
+  for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+    for (int tj = 0; tj < 2; tj++) {
+      const int64_t col = j0 + tj * 16 + li;
+      if (col >= n_dense) continue;
+      const int64_t row = i0 + ti * 16 + lk * 4;
+      OutT o[4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        float v = acc[ti][tj][r] * scale;
+        if (bias) v += to_float(bias[row + r]);
+        o[r] = from_float<OutT>(apply_act(v, act));
+      }
+      if constexpr (C_JMAJOR) {
+        *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
+      }
+    }
+}
+
+template <typename T, typename OutT>
+int launch_general(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
+                   int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
+  dim3 grid((unsigned)((n_dense + 63) / 64), (unsigned)((n_sparse + 63) / 64));
+  const bool kc = b_layout == TF24_ROW_MAJOR, jm = c_layout == TF24_COL_MAJOR;
+#define TF24_GO(KC, JM)                                                                                              \
+  hipLaunchKernelGGL((spmm_general<T, OutT, KC, JM>), grid, dim3(256), 0, s, (const uint8_t*)av, (const uint8_t*)am, \
+                     n_sparse, k, (const T*)b, ldb, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act)
+  if (kc && jm) TF24_GO(true, true);
+  else if (kc) TF24_GO(true, false);
+  else if (jm) TF24_GO(false, true);
+  else TF24_GO(false, false);
+#undef TF24_GO
+  return check_launch("tf24_spmm");
+}
+
+template <typename T>
+int dispatch_out(int out_dtype, const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout,
+                 int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
+                 hipStream_t s) {
+  switch (out_dtype) {
+    case TF24_F16: return launch_general<T, f16_t>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_BF16: return launch_general<T, bf16_t>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_F32: return launch_general<T, float>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+  }
+  return fail(TF24_ERR_DTYPE, "tf24_spmm: unsupported output dtype %d", out_dtype);
+}
+
+}  // namespace
+}  // namespace tf24
+
+extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_layout, int64_t ldb, int64_t n_dense,
+                                  int out_dtype, int c_layout, int64_t ldc, int activation) {
+  using namespace tf24;
+  const char* fn = "tf24_spmm";
+  if (dtype != TF24_F16 && dtype != TF24_BF16 && dtype != TF24_E4M3) return fail(TF24_ERR_DTYPE, "%s: unsupported operand dtype %d", fn, dtype);
+  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && out_dtype != TF24_F32) return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
+  const bool eight = dtype == TF24_E4M3;
+  const int64_t kmult = eight ? 128 : 64, dmult = eight ? 16 : 8;
+  if (n_sparse <= 0 || n_sparse % 32) return fail(TF24_ERR_SHAPE, "%s: sparse operand rows %lld must be a positive multiple of 32", fn, (long long)n_sparse);
+  if (k <= 0 || k % kmult) return fail(TF24_ERR_SHAPE, "%s: inner dimension %lld must be a positive multiple of %lld", fn, (long long)k, (long long)kmult);
+  if (n_dense <= 0 || n_dense % dmult) return fail(TF24_ERR_SHAPE, "%s: dense operand extent %lld must be a positive multiple of %lld", fn, (long long)n_dense, (long long)dmult);
+  if (b_layout != TF24_ROW_MAJOR && b_layout != TF24_COL_MAJOR) return fail(TF24_ERR_ARG, "%s: bad b_layout %d", fn, b_layout);
+  if (c_layout != TF24_ROW_MAJOR && c_layout != TF24_COL_MAJOR) return fail(TF24_ERR_ARG, "%s: bad c_layout %d", fn, c_layout);
+  const int64_t bext = b_layout == TF24_ROW_MAJOR ? k : n_dense;
+  if (ldb < bext || ldb % dmult) return fail(TF24_ERR_STRIDE, "%s: ldb %lld must be >= %lld and a multiple of %lld", fn, (long long)ldb, (long long)bext, (long long)dmult);
+  const int64_t cext = c_layout == TF24_ROW_MAJOR ? n_dense : n_sparse;
+  if (ldc < cext || ldc % 4) return fail(TF24_ERR_STRIDE, "%s: ldc %lld must be >= %lld and a multiple of 4", fn, (long long)ldc, (long long)cext);
+  if (activation < TF24_ACT_NONE || activation > TF24_ACT_SILU) return fail(TF24_ERR_ARG, "%s: bad activation %d", fn, activation);
+  return TF24_OK;
+}
+
+extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int dtype, int64_t n_sparse, int64_t k,
+                         const void* b, int b_layout, int64_t ldb, int64_t n_dense,
+                         void* c, int out_dtype, int c_layout, int64_t ldc,
+                         const void* bias, float scale, int activation, void* stream) {
+  using namespace tf24;
+  int rc = tf24_spmm_validate(dtype, n_sparse, k, b_layout, ldb, n_dense, out_dtype, c_layout, ldc, activation);
+  if (rc) return rc;
+  if (!a_values || !a_meta || !b || !c) return fail(TF24_ERR_ARG, "tf24_spmm: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+  }
+}

@@ -1,0 +1,168 @@
+// Shared device/host helpers for the gfx950 2:4 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tf24.h"
+
+namespace tf24 {
+
+// ---------------------------------------------------------------- error reporting (host)
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+// ---------------------------------------------------------------- element types
+struct f16_t { uint16_t bits; };
+struct bf16_t { uint16_t bits; };
+struct e4m3_t { uint8_t bits; };
+
+template <typename T> struct dtype_of;
+template <> struct dtype_of<float> { static constexpr int value = TF24_F32; };
+template <> struct dtype_of<f16_t> { static constexpr int value = TF24_F16; };
+template <> struct dtype_of<bf16_t> { static constexpr int value = TF24_BF16; };
+template <> struct dtype_of<e4m3_t> { static constexpr int value = TF24_E4M3; };
+template <> struct dtype_of<uint8_t> { static constexpr int value = TF24_U8; };
+
+__host__ __device__ inline int dtype_size(int dt) {
+  return dt == TF24_F32 ? 4 : (dt == TF24_F16 || dt == TF24_BF16) ? 2 : 1;
+}
+
+// ---------------------------------------------------------------- conversions to float (exact)
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(f16_t v) {
+  return (float)__builtin_bit_cast(_Float16, v.bits);
+}
+__device__ __forceinline__ float to_float(bf16_t v) {
+  return __builtin_bit_cast(float, (uint32_t)v.bits << 16);
+}
+__device__ __forceinline__ float to_float(uint8_t v) { return (float)v; }
+
+// ---------------------------------------------------------------- conversions from float
+// round-to-nearest-even everywhere, like a plain tensor cast
+template <typename T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) {
+  return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};
+}
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)((u >> 16) | 0x40)};  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return bf16_t{(uint16_t)(u >> 16)};
+}
+// OCP e4m3fn (bias 7, no inf, 0x7f = NaN, max 448): values that round past 448 become NaN,
+// exactly like the bit pattern arithmetic of a round-to-nearest-even narrowing.
+__host__ __device__ inline uint8_t float_to_e4m3(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  uint32_t sign = (u >> 24) & 0x80u;
+  u &= 0x7fffffffu;
+  uint32_t r;
+  if (u >= 0x43f00000u) {            // |f| >= 480, inf, NaN
+    r = 0x7fu;
+  } else if (u < 0x3c800000u) {      // |f| < 2^-6: subnormal result, multiples of 2^-9
+    float a = __builtin_bit_cast(float, u) + 16384.0f;   // ulp(16384) * 2^-23.. aligns 2^-9 to bit 0
+    r = __builtin_bit_cast(uint32_t, a) - 0x46800000u;   // 16384.0f == 0x46800000
+  } else {
+    uint32_t odd = (u >> 20) & 1u;
+    u += 0x7ffffu + odd;             // RTNE at bit 20
+    r = (u >> 20) - ((127u - 7u) << 3);
+  }
+  return (uint8_t)(r | sign);
+}
+template <> __device__ __forceinline__ e4m3_t from_float<e4m3_t>(float f) { return e4m3_t{float_to_e4m3(f)}; }
+
+__host__ __device__ inline float e4m3_to_float(uint8_t b) {
+  uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+  uint32_t e = (b >> 3) & 0xfu, m = b & 7u;
+  float v;
+  if (e == 0) v = (float)m * 0.001953125f;                                    // m * 2^-9
+  else if (e == 15 && m == 7) v = __builtin_bit_cast(float, 0x7fc00000u);     // NaN
+  else v = __builtin_bit_cast(float, ((e + 120u) << 23) | (m << 20));
+  return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) | sign);
+}
+__device__ __forceinline__ float to_float(e4m3_t v) { return e4m3_to_float(v.bits); }
+
+// ---------------------------------------------------------------- vector loads/stores
+template <int BYTES> struct vec_bytes;
+template <> struct vec_bytes<2> { using type = uint16_t; };
+template <> struct vec_bytes<4> { using type = uint32_t; };
+template <> struct vec_bytes<8> { using type = uint2; };
+template <> struct vec_bytes<16> { using type = uint4; };
+template <> struct vec_bytes<32> { struct alignas(16) type { uint4 a, b; }; };
+
+// load N elements of T (N*sizeof(T) in {2,4,8,16,32} bytes, naturally aligned)
+template <typename T, int N>
+struct Pack {
+  T v[N];
+  __device__ __forceinline__ void load(const T* p) {
+    using V = typename vec_bytes<sizeof(T) * N>::type;
+    *reinterpret_cast<V*>(v) = *reinterpret_cast<const V*>(p);
+  }
+  __device__ __forceinline__ void store(T* p) const {
+    using V = typename vec_bytes<sizeof(T) * N>::type;
+    *reinterpret_cast<V*>(p) = *reinterpret_cast<const V*>(v);
+  }
+};
+
+// ---------------------------------------------------------------- 2:4 group math
+// Magnitude mask: bit i set = element i kept.  Six strict compares of |x|; ties keep the
+// larger index (all equal -> elements 2 and 3).
+__device__ __forceinline__ uint32_t magnitude_mask4(float x0, float x1, float x2, float x3) {
+  float a = __builtin_fabsf(x0), b = __builtin_fabsf(x1), c = __builtin_fabsf(x2), d = __builtin_fabsf(x3);
+  bool x1_ = a > b, x2_ = a > c, x3_ = a > d, x4_ = b > c, x5_ = b > d, x6_ = c > d;
+  bool m0 = (x2_ & x3_) | (x1_ & x2_) | (x1_ & x3_);
+  bool m1 = (!x1_ & x5_) | (x4_ & x5_) | (!x1_ & x4_);
+  bool m2 = (!x2_ & !x4_) | (!x2_ & x6_) | (!x4_ & x6_);
+  bool m3 = (!x3_ & !x5_) | (!x3_ & !x6_) | (!x5_ & !x6_);
+  return (uint32_t)m0 | ((uint32_t)m1 << 1) | ((uint32_t)m2 << 2) | ((uint32_t)m3 << 3);
+}
+
+// mask bits -> nibble pos0 | pos1<<2 (the 16-row table: masks with other than two bits set
+// are mapped as the reference's boolean minimisation maps them)
+__device__ __forceinline__ uint32_t encode_nibble(uint32_t mbits) {
+  bool m0 = mbits & 1, m1 = mbits & 2, m2 = mbits & 4;
+  bool bit0 = !m0 & m1;
+  bool bit1 = !m0 & !m1;
+  bool bit2 = bit1 | !m2;
+  bool bit3 = bit0 | !m1 | m2;
+  return (uint32_t)bit0 | ((uint32_t)bit1 << 1) | ((uint32_t)bit2 << 2) | ((uint32_t)bit3 << 3);
+}
+
+template <typename T>
+__device__ __forceinline__ T select4(uint32_t pos, T v0, T v1, T v2, T v3) {
+  T lo = (pos & 1) ? v1 : v0;
+  T hi = (pos & 1) ? v3 : v2;
+  return (pos & 2) ? hi : lo;
+}
+
+// MVUE24 of one group in float32, in the reference's operation order (no contraction).
+// Outputs the rescaled values y_i = x_i / p_i and the kept-mask bits.
+__device__ __forceinline__ uint32_t mvue4(float x0, float x1, float x2, float x3, float r0, float r1,
+                                          float& y0, float& y1, float& y2, float& y3) {
+  const float eps = 1.19209e-07f;
+  float a0 = __builtin_fabsf(x0) + eps, a1 = __builtin_fabsf(x1) + eps;
+  float a2 = __builtin_fabsf(x2) + eps, a3 = __builtin_fabsf(x3) + eps;
+  float sum = ((a0 + a1) + a2) + a3;
+  float t0 = a0 / sum, t1 = a1 / sum, t2 = a2 / sum, t3 = a3 / sum;
+  float s0 = sum - a0, s1 = sum - a1, s2 = sum - a2, s3 = sum - a3;
+  float k0 = t0 / s0, k1 = t1 / s1, k2 = t2 / s2, k3 = t3 / s3;
+  float k = ((k0 + k1) + k2) + k3;
+  float p0 = t0 + a0 * (k - k0), p1 = t1 + a1 * (k - k1);
+  float p2 = t2 + a2 * (k - k2), p3 = t3 + a3 * (k - k3);
+  bool m0 = r0 <= t0;
+  bool m1 = (r0 <= (t0 + t1)) & !m0;
+  bool m2 = (r0 <= ((t0 + t1) + t2)) & !m1 & !m0;
+  bool m3 = !m2 & !m1 & !m0;
+  float d0 = m0 ? 0.0f : a0, d1 = m1 ? 0.0f : a1, d2 = m2 ? 0.0f : a2, d3 = m3 ? 0.0f : a3;
+  float dsum = ((d0 + d1) + d2) + d3;
+  float t = r1 * dsum;
+  bool e0 = t <= d0;
+  bool e1 = (t <= (d0 + d1)) & !e0;
+  bool e2 = (t <= ((d0 + d1) + d2)) & !e1 & !e0;
+  bool e3 = !e2 & !e1 & !e0;
+  y0 = x0 / p0; y1 = x1 / p1; y2 = x2 / p2; y3 = x3 / p3;
+  return (uint32_t)(m0 | e0) | ((uint32_t)(m1 | e1) << 1) | ((uint32_t)(m2 | e2) << 2) | ((uint32_t)(m3 | e3) << 3);
+}
+
+}  // namespace tf24

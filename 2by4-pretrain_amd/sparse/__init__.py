@@ -1,0 +1,21 @@
+"""`sparse`: drop-in for the 2:4 sparse hot path of huyz2023/2by4-pretrain on MI355X (gfx950).
+
+Same names as the reference package (sparse/__init__.py:1-25) for everything on the 2:4 path;
+every operator runs a hand-written HIP kernel from lib2by4_gfx950.so and raises if that library
+is missing -- there is no CPU or PyTorch fallback.
+"""
+from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured
+from .transposable_semi_structured import TransposableSparse, mask_select
+from .decay import masked_add_
+from .dense_ops import (soft_threshold24, sparse24, MVUE24_approx,
+                        soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton)
+from .sparse_linear_transpose import SparseLinearTranspose, sparse_linear_transpose
+
+__all__ = [
+    "SparseSemiStructuredTensor", "to_sparse_semi_structured",
+    "TransposableSparse", "mask_select",
+    "masked_add_",
+    "soft_threshold24", "sparse24", "MVUE24_approx",
+    "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
+    "SparseLinearTranspose", "sparse_linear_transpose",
+]

@@ -1,0 +1,313 @@
+"""SparseSemiStructuredTensor / to_sparse_semi_structured on the gfx950 2:4 library.
+
+Mirrors the public surface of sparse/semi_structured.py of huyz2023/2by4-pretrain (class
+:33-572, factory :575-631): same constructor arguments, attributes, dispatch rules and error
+behaviour.  Differences, all deliberate:
+  * one backend (hand-written HIP on SMFMAC); `_FORCE_CUTLASS` / `_FUSE_TRANSPOSE` are kept as
+    inert attributes, `compressed_tensor_cusparselt` is always None;
+  * `meta_tensor_cutlass` holds the CANONICAL row-major nibble metadata (what one SMFMAC lane
+    consumes), not CUTLASS's reordered layout; `indices_cutlass()` exports the reordered form;
+  * compressed values are always row-major [m, k/2], also for column-major inputs (`W.T`);
+  * MVUE24 takes its uniforms from an optional `rand` tensor (drawn with torch.rand when omitted);
+  * `addmm` / `linear` with a bias work (the reference passes a wrong keyword there).
+"""
+import warnings
+from collections import namedtuple
+from typing import Any, Optional
+
+import torch
+
+from . import _native as N
+
+__all__ = ["SparseSemiStructuredTensor", "to_sparse_semi_structured"]
+
+_Config = namedtuple("_SEMI_STRUCTURED_SPARSE_CONFIG",
+                     "compression_factor sparse_min_rows sparse_min_cols dense_min_rows dense_min_cols")
+# semi_structured.py:24-30 of the reference, restricted to what SMFMAC kernels exist for
+_DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG = {
+    torch.float8_e4m3fn: _Config(10, 32, 128, 16, 16),
+    torch.float16: _Config(9, 32, 64, 8, 8),
+    torch.bfloat16: _Config(9, 32, 64, 8, 8),
+}
+
+
+def _indices_dtype(values_dtype):
+    if values_dtype == torch.float8_e4m3fn:
+        return torch.int32
+    if values_dtype in (torch.float16, torch.bfloat16):
+        return torch.int16
+    raise RuntimeError(f"Datatype {values_dtype}  is not supported!")
+
+
+def _compress(original, dtype, MVUE24, mask, rand):
+    """One allocation of numel*cf/16 elements: values first, metadata in the tail
+    (reference :215-243); then the HIP prune+compress kernel."""
+    m, n = original.shape
+    cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[dtype]
+    buf = torch.empty((original.nelement() * cfg.compression_factor // 16,), dtype=dtype, device=original.device)
+    values = buf[: m * n // 2].view(m, n // 2)
+    meta = buf[m * n // 2:].view(_indices_dtype(dtype)).view(m, -1)
+
+    dense = N.as_matrix(original)
+    layout, ld = N.layout_of(dense)
+    mode, mask_t, rand_t = N.PRUNE_MAGNITUDE, None, None
+    mask_ld = rand_ld = 0
+    mask_code = N.U8
+    if mask is not None:
+        if mask.shape != original.shape:
+            raise RuntimeError(f"mask shape {tuple(mask.shape)} does not match tensor shape {tuple(original.shape)}")
+        mode = N.PRUNE_MASK
+        mask_t = N.as_matrix(mask, like=dense)
+        mask_ld = N.layout_of(mask_t)[1]
+        mask_code = N.dtype_code(mask_t.dtype)
+    elif MVUE24:
+        mode = N.PRUNE_MVUE
+        if rand is None:
+            rand = torch.empty_strided(dense.shape, dense.stride(), dtype=torch.float32, device=dense.device).uniform_()
+        if rand.shape != original.shape:
+            raise RuntimeError(f"rand shape {tuple(rand.shape)} does not match tensor shape {tuple(original.shape)}")
+        rand_t = N.as_matrix(rand.float(), like=dense)
+        rand_ld = N.layout_of(rand_t)[1]
+    N.check(N.lib().tf24_prune_compress(
+        dense.data_ptr(), N.dtype_code(dense.dtype), layout, ld, m, n, mode,
+        N.ptr(mask_t), mask_code, mask_ld, N.ptr(rand_t), rand_ld,
+        values.data_ptr(), N.dtype_code(dtype), meta.data_ptr(), N.stream_ptr()))
+    return values, meta
+
+
+def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, activation=N.ACT_NONE):
+    """sparse_first: out = S @ dense  (S [n,k], dense [k,j])  -> [n, j]
+       otherwise   : out = dense @ S^T (dense [j,k])          -> [j, n]"""
+    values, meta = sparse.sparse_tensor_cutlass, sparse.meta_tensor_cutlass
+    n, half_k = values.shape
+    k = 2 * half_k
+    if dense.dtype != values.dtype:
+        raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
+    dense = N.as_matrix(dense)
+    lay, ld = N.layout_of(dense)
+    if sparse_first:
+        kk, j = dense.shape
+        b_layout = N.COL_MAJOR if lay == N.ROW_MAJOR else N.ROW_MAJOR   # k strided when the [k,j] tensor is row-major
+        c_layout, out_shape = N.ROW_MAJOR, (n, j)
+    else:
+        j, kk = dense.shape
+        b_layout = N.ROW_MAJOR if lay == N.ROW_MAJOR else N.COL_MAJOR
+        c_layout, out_shape = N.COL_MAJOR, (j, n)
+    if kk != k:
+        raise RuntimeError(f"inner dimensions do not match: sparse operand has k={k}, dense operand {tuple(dense.shape)}")
+    if out_dtype is None:
+        out_dtype = torch.float32 if values.dtype == torch.float8_e4m3fn else values.dtype
+    out = torch.empty(out_shape, dtype=out_dtype, device=dense.device)
+    if bias is not None:
+        bias = bias.to(out_dtype).contiguous()
+        if bias.numel() != n:
+            raise RuntimeError(f"bias must have {n} elements, got {bias.numel()}")
+    N.check(N.lib().tf24_spmm(
+        values.data_ptr(), meta.data_ptr(), N.dtype_code(values.dtype), n, k,
+        dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.dtype_code(out_dtype), c_layout, out.stride(0),
+        N.ptr(bias), float(scale), activation, N.stream_ptr()))
+    return out
+
+
+class SparseSemiStructuredTensor(torch.Tensor):
+    """2:4 semi-structured sparse matrix as a wrapper tensor subclass: logically the dense
+    [m, k] matrix, physically `sparse_tensor_cutlass` (kept values [m, k/2]) and
+    `meta_tensor_cutlass` (2-bit positions, int16 [m, k/16] or int32 [m, k/32]).
+
+    Supported ops: detach, t, mm, addmm, linear, values, indices; the sparse operand must be the
+    first and untransposed or the second and transposed argument."""
+
+    _FUSE_TRANSPOSE = False
+    _FORCE_CUTLASS = True
+    _PROTOTYPE_WARNING_SHOWN = False
+    # output dtype of fp8 products (the reference's CUTLASS path returns float32)
+    _FP8_OUT_DTYPE = torch.float32
+
+    @staticmethod
+    def __new__(cls, original_tensor: Optional[torch.Tensor], original_shape: Optional[torch.Size] = None,
+                compressed_tensor_cusparselt: Optional[torch.Tensor] = None,
+                sparse_tensor_cutlass: Optional[torch.Tensor] = None,
+                meta_tensor_cutlass: Optional[torch.Tensor] = None, transposed: bool = False,
+                MVUE24: bool = False, mask: Optional[torch.Tensor] = None,
+                dtype: Optional[torch.dtype] = None, rand: Optional[torch.Tensor] = None):
+        assert compressed_tensor_cusparselt is None or (sparse_tensor_cutlass is None and meta_tensor_cutlass is None)
+        if not cls._PROTOTYPE_WARNING_SHOWN:
+            warnings.warn(
+                "The PyTorch API of SparseSemiStructuredTensor is in prototype stage and will change in the "
+                "near future. Please open a Github issue for features requests and see our documentation on "
+                "the torch.sparse module for further information about the project.", UserWarning)
+            cls._PROTOTYPE_WARNING_SHOWN = True
+        if original_tensor is not None:
+            previous, original_shape = original_tensor, original_tensor.shape
+        elif compressed_tensor_cusparselt is not None:
+            previous = compressed_tensor_cusparselt
+        elif sparse_tensor_cutlass is not None:
+            previous = sparse_tensor_cutlass
+        else:
+            raise ValueError("All of the tensor arguments are None!")
+        return torch.Tensor._make_wrapper_subclass(
+            cls, original_shape, device=previous.device, dtype=previous.dtype if dtype is None else dtype,
+            layout=previous.layout, requires_grad=False)
+
+    def __init__(self, original_tensor: Optional[torch.Tensor], original_shape: Optional[torch.Size] = None,
+                 compressed_tensor_cusparselt: Optional[torch.Tensor] = None,
+                 sparse_tensor_cutlass: Optional[torch.Tensor] = None,
+                 meta_tensor_cutlass: Optional[torch.Tensor] = None, transposed: bool = False,
+                 MVUE24: bool = False, mask: Optional[torch.Tensor] = None,
+                 dtype: Optional[torch.dtype] = torch.float16, rand: Optional[torch.Tensor] = None) -> None:
+        if original_tensor is not None:
+            if not original_tensor.is_cuda:
+                raise RuntimeError(f"Error original_tensor.device= {original_tensor.device} is not supported! "
+                                   "Only CUDA tensors are currently supported.")
+            if original_tensor.dim() != 2:
+                raise RuntimeError(f"Error original_tensor.dim = {original_tensor.dim()} is not supported! "
+                                   "Only 2d tensors are currently supported.")
+            if dtype not in _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG:
+                raise RuntimeError(f"Error dtype {dtype} is not a supported dtype! "
+                                   f"dtype must be one of: {list(_DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG)}")
+            m, n = original_tensor.shape
+            cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[dtype]
+            if m < cfg.sparse_min_rows or m % cfg.sparse_min_rows or n < cfg.sparse_min_cols or n % cfg.sparse_min_cols:
+                raise RuntimeError(f"Error original_tensor.shape {original_tensor.shape} is not supported! "
+                                   "Both dimensions must be larger or equal than and a multiple of "
+                                   f"({cfg.sparse_min_rows}, {cfg.sparse_min_cols})")
+            if mask is not None and MVUE24:
+                raise RuntimeError("Error using MVUE24 with mask is not supported! ")
+            compressed_tensor_cusparselt = None
+            sparse_tensor_cutlass, meta_tensor_cutlass = _compress(original_tensor, dtype, MVUE24, mask, rand)
+        self.original_tensor = None
+        self.compressed_tensor_cusparselt = compressed_tensor_cusparselt
+        self.sparse_tensor_cutlass = sparse_tensor_cutlass
+        self.meta_tensor_cutlass = meta_tensor_cutlass
+        self.transposed = transposed
+        self.original_shape = original_shape
+
+    def __tensor_flatten__(self):
+        return ["sparse_tensor_cutlass", "meta_tensor_cutlass"], (self.original_shape, self.transposed)
+
+    @staticmethod
+    def __tensor_unflatten__(inner_tensors, meta, outer_size, outer_stride):
+        original_shape, transposed = meta
+        if len(inner_tensors) != 2:
+            raise RuntimeError(f"Expected 2 inner tensors but got {len(inner_tensors)}")
+        return SparseSemiStructuredTensor(
+            None, original_shape=original_shape, sparse_tensor_cutlass=inner_tensors["sparse_tensor_cutlass"],
+            meta_tensor_cutlass=inner_tensors["meta_tensor_cutlass"], transposed=transposed)
+
+    def __repr__(self) -> str:  # type: ignore[override]
+        return (f"SparseSemiStructuredTensor(shape={self.shape}, transposed={self.transposed}"
+                f"values={self.values()}metadata={self.indices()})")
+
+    __torch_function__ = torch._C._disabled_torch_function_impl
+
+    def _clone_view(self, shape, transposed):
+        return SparseSemiStructuredTensor(
+            None, original_shape=shape, sparse_tensor_cutlass=self.sparse_tensor_cutlass,
+            meta_tensor_cutlass=self.meta_tensor_cutlass, transposed=transposed, dtype=self.dtype)
+
+    def _pad_tensor_for_matmul(self, original_tensor: torch.Tensor) -> torch.Tensor:
+        """Zero-pads a 2-d dense operand to the multiples the kernel wants (reference :351-368)."""
+        assert original_tensor.dim() == 2
+        m, n = original_tensor.shape
+        cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[original_tensor.dtype]
+        to_pad_m = -m % cfg.dense_min_rows
+        to_pad_n = -n % cfg.dense_min_cols
+        if to_pad_m or to_pad_n:
+            return torch.nn.functional.pad(original_tensor, (0, to_pad_n, 0, to_pad_m))
+        return original_tensor
+
+    def _out_dtype(self):
+        return self._FP8_OUT_DTYPE if self.dtype == torch.float8_e4m3fn else None
+
+    @classmethod
+    def __torch_dispatch__(cls, func, types, args, kwargs) -> Any:
+        if func is torch.ops.aten.detach.default:
+            return args[0]._clone_view(args[0].shape, args[0].transposed)
+
+        # the compressed form cannot be transposed; only the number of transposes is tracked
+        if func is torch.ops.aten.t.default:
+            s = args[0]
+            return s._clone_view(torch.Size([s.shape[1], s.shape[0]]), not s.transposed)
+
+        if func is torch.ops.aten.addmm.default:
+            bias, input_A, input_B = args
+            # F.linear(x) = addmm(bias, x, W.t()) = (W x' + b')'
+            if isinstance(input_B, cls) and input_B.transposed:
+                row, _ = input_A.shape
+                padded = input_B._pad_tensor_for_matmul(input_A)
+                return _spmm(input_B, padded, False, bias=bias, out_dtype=input_B._out_dtype())[:row, :]
+
+        if func is torch.ops.aten.mm.default:
+            input_A, input_B = args
+            if isinstance(input_A, cls) and not input_A.transposed:          # first operand sparse
+                _, col = input_B.shape
+                padded = input_A._pad_tensor_for_matmul(input_B)
+                return _spmm(input_A, padded, True, out_dtype=input_A._out_dtype())[:, :col]
+            if isinstance(input_B, cls) and input_B.transposed:              # second operand sparse
+                row, _ = input_A.shape
+                padded = input_B._pad_tensor_for_matmul(input_A)
+                return _spmm(input_B, padded, False, out_dtype=input_B._out_dtype())[:row, :]
+
+        # inference mode does not decompose linear into t + addmm
+        if func is torch.ops.aten.linear.default:
+            input_tensor, weight, bias = args
+            if isinstance(weight, cls):
+                shape = input_tensor.shape
+                x2d = input_tensor.reshape(-1, shape[-1])
+                row, _ = x2d.shape
+                padded = weight._pad_tensor_for_matmul(x2d)
+                res = _spmm(weight, padded, False, bias=bias, out_dtype=weight._out_dtype())
+                return res[:row, :].view(*shape[:-1], -1)
+
+        if func is torch.ops.aten.values.default:
+            return args[0].sparse_tensor_cutlass.detach()
+
+        if func is torch.ops.aten.indices.default:
+            return args[0].meta_tensor_cutlass
+
+        error_string = "\n".join([f"func {func} with args: "] + [f"arg{i}: {arg}" for i, arg in enumerate(args)])
+        raise NotImplementedError(error_string)
+
+    def to_dense(self):
+        """Decompress to a dense [m, k] tensor of the value dtype (reference :554-572)."""
+        values, meta = self.sparse_tensor_cutlass, self.meta_tensor_cutlass
+        m, half_k = values.shape
+        out = torch.empty((m, 2 * half_k), dtype=values.dtype, device=values.device)
+        N.check(N.lib().tf24_decompress(values.data_ptr(), N.dtype_code(values.dtype), meta.data_ptr(), m, 2 * half_k,
+                                        out.data_ptr(), N.stream_ptr()))
+        return out
+
+    def indices_cutlass(self):
+        """Metadata in the CUTLASS-reordered layout the reference's `indices()` returns
+        (reorder_meta + ColumnMajorInterleaved<2>; csrc .cu:826-851)."""
+        meta = self.meta_tensor_cutlass
+        m, ncols = meta.shape
+        group, inter = (32, 4) if meta.dtype == torch.int16 else (16, 2)
+        r = torch.arange(m, device=meta.device).view(-1, 1).expand(m, ncols)
+        c = torch.arange(ncols, device=meta.device).view(1, -1).expand(m, ncols)
+        dr = r // group * group + (r % 8) * inter + (r % group) // 8
+        tr = ((dr % 2 == 0) & (c % 2 == 1)).long()
+        bl = ((dr % 2 == 1) & (c % 2 == 0)).long()
+        dr, dc = dr + tr - bl, c - tr + bl
+        dest = (dc // 2) * m * 2 + dr * 2 + dc % 2
+        out = torch.empty_like(meta).view(-1)
+        out[dest.reshape(-1)] = meta.reshape(-1)
+        return out.view(m, ncols)
+
+
+def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = False, MVUE24: bool = False,
+                              mask: Optional[torch.Tensor] = None, dtype: torch.dtype = torch.float16,
+                              rand: Optional[torch.Tensor] = None) -> SparseSemiStructuredTensor:
+    """Dense [m, k] device tensor -> SparseSemiStructuredTensor, pruned 2:4 along k.
+
+    Without `mask`/`MVUE24` the two largest |x| of every 4 are kept (ties: larger index);
+    `mask` (same shape, nonzero = keep) selects explicitly; `MVUE24=True` samples the
+    minimum-variance unbiased estimator, taking its uniforms from `rand` (same shape, U[0,1);
+    drawn with torch's generator when omitted).  `dtype` is the value dtype of the result
+    (float16, bfloat16 or float8_e4m3fn).  Rows must be a multiple of 32, columns of 64
+    (128 for float8).  Same signature as the reference's factory (semi_structured.py:575-631)
+    plus `rand`.
+    """
+    return SparseSemiStructuredTensor(
+        original_tensor, original_shape=original_tensor.shape, transposed=transposed,
+        MVUE24=MVUE24, mask=mask, dtype=dtype, rand=rand)

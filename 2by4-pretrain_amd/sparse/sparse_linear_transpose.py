@@ -1,0 +1,87 @@
+"""SparseLinearTranspose / sparse_linear_transpose: 2:4 sparse training linear layer.
+
+The reference defines these only in its README (README.md:125-200): an nn.Linear whose
+weight carries a transposable 2:4 mask (refreshed every `freq` optimizer steps), two compressed
+copies (W and W.T) rebuilt once per optimizer step, and an autograd function computing
+    y  = x . W_sparse^T           (2:4 spMM)
+    dX = dY . W_sparse_T^T        (2:4 spMM on the transposed copy)
+    dW = MVUE24(dY^T) . x         (2:4 spMM with the gradient pruned along the token axis)
+    db = sum(dY)
+State lives as attributes on the weight Parameter, exactly as in the README: freq, cnt, counter,
+step, mask, weight_sparse, weight_sparse_T, mode.
+"""
+import torch
+import torch.nn.functional as F
+from torch import autograd, nn
+from torch.amp import custom_bwd, custom_fwd
+
+from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured
+from .transposable_semi_structured import TransposableSparse
+
+__all__ = ["SparseLinearTranspose", "sparse_linear_transpose"]
+
+
+class sparse_linear_transpose(autograd.Function):
+    @staticmethod
+    @custom_fwd(device_type="cuda", cast_inputs=torch.float16)
+    def forward(ctx, input, weight, weight_sparse, weight_sparse_T, bias):
+        ctx.save_for_backward(input, weight_sparse_T, bias)
+        ctx.shape = input.shape
+        input = input.view(-1, input.shape[-1])
+        output = torch.mm(input, weight_sparse.t())
+        if bias is None:
+            return output.view(*ctx.shape[:-1], -1)
+        return output.view(*ctx.shape[:-1], -1) + bias
+
+    @staticmethod
+    @custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        input, weight_T, bias = ctx.saved_tensors
+        grad_input = grad_weight = grad_bias = None
+        if grad_output.stride() == (0,) * grad_output.dim():       # expanded scalar gradient
+            grad_output = torch.ones_like(grad_output)
+        grad_output = grad_output.reshape(-1, grad_output.shape[-1])
+        if ctx.needs_input_grad[0]:
+            grad_input = torch.mm(grad_output, weight_T.t()).view(ctx.shape)
+        if ctx.needs_input_grad[1]:
+            input = input.view(-1, input.shape[-1])
+            grad_weight = torch.mm(to_sparse_semi_structured(grad_output.t(), MVUE24=True, dtype=grad_output.dtype), input)
+        if ctx.needs_input_grad[4]:
+            grad_bias = grad_output.sum(0)
+        return grad_input, grad_weight, None, None, grad_bias
+
+
+class SparseLinearTranspose(nn.Linear):
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, func=lambda step: 'dense', **kwargs):
+        super().__init__(in_features, out_features, bias=bias, **kwargs)
+        self.weight.freq = 40      # mask refresh period, in optimizer steps
+        self.weight.cnt = 0        # forward passes since the last optimizer step
+        self.weight.counter = 0    # optimizer steps
+        self.weight.step = 0       # forward passes in training mode
+        self.weight.mask = torch.ones_like(self.weight, dtype=torch.bool)
+        self.weight.weight_sparse = None
+        self.weight.weight_sparse_T = None
+        self.weight.mode = 'sparse'
+        self.func = func
+        self.transposable_sparse = TransposableSparse(abs=True)
+        SparseSemiStructuredTensor._FORCE_CUTLASS = True
+
+    def forward(self, x):
+        w = self.weight
+        if w.mode == 'dense':
+            x = F.linear(x, w, self.bias)
+        else:
+            w.mask = w.mask.to(device=w.device)
+            if w.counter % w.freq == 0 and w.cnt == 0:
+                _, w.mask = self.transposable_sparse(w)
+            if w.cnt == 0:
+                w.weight_sparse = to_sparse_semi_structured(w, mask=w.mask, dtype=torch.float16)
+                w.weight_sparse_T = to_sparse_semi_structured(w.T, mask=w.mask.T, dtype=torch.float16)
+            with torch.autocast(device_type='cuda', dtype=torch.float16):
+                x = sparse_linear_transpose.apply(x, w, w.weight_sparse, w.weight_sparse_T, self.bias)
+        if self.training:
+            if w.cnt == 0:
+                w.counter += 1
+            w.step += 1
+            w.cnt += 1
+        return x

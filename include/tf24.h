@@ -1,0 +1,162 @@
+/*
+ * tf24.h -- C ABI of lib2by4_gfx950.so: the 2:4 semi-structured sparse hot path of
+ * huyz2023/2by4-pretrain, hand-written for MI355X (gfx950 / CDNA4).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer (HIP) unless the name ends in _host.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Nothing here
+ *     allocates, frees or synchronises: the caller owns every buffer, work is only enqueued.
+ *   - Return value: TF24_OK or a negative tf24_status; tf24_last_error() returns a
+ *     thread-local human readable message for the last failure on the calling thread.
+ *   - A logical [m,k] matrix is described by (layout, ld):
+ *       TF24_ROW_MAJOR element (r,c) at r*ld + c,   TF24_COL_MAJOR element (r,c) at c*ld + r.
+ *   - "group" = 4 consecutive elements along k.  Compressed values are always written
+ *     row-major [m, k/2]; metadata is the canonical nibble stream: for each group
+ *     pos0 | pos1<<2 (pos0 < pos1 = positions of the two kept elements), packed LSB-first
+ *     into int16 [m, k/16] for 16-bit values or int32 [m, k/32] for 8-bit values.  One int16
+ *     is exactly the index operand of one lane of V_SMFMAC_F32_16X16X64_{F16,BF16}; one int32
+ *     that of V_SMFMAC_F32_16X16X128_FP8_FP8.
+ *
+ * Each entry point names the reference interface (huyz2023/2by4-pretrain) it replaces.
+ */
+#ifndef TF24_H
+#define TF24_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  TF24_OK = 0,
+  TF24_ERR_SHAPE = -1,   /* dimension not supported (multiples, minima) */
+  TF24_ERR_DTYPE = -2,   /* dtype or dtype combination not supported */
+  TF24_ERR_STRIDE = -3,  /* leading dimension / alignment not supported */
+  TF24_ERR_LAUNCH = -4,  /* HIP reported an error at launch */
+  TF24_ERR_ARG = -5      /* null pointer, bad enum, contradictory arguments */
+} tf24_status;
+
+typedef enum {
+  TF24_F32 = 0,
+  TF24_F16 = 1,
+  TF24_BF16 = 2,
+  TF24_E4M3 = 3, /* OCP float8 e4m3fn */
+  TF24_U8 = 4    /* bytes: bool masks (nonzero = kept) */
+} tf24_dtype;
+
+typedef enum { TF24_ROW_MAJOR = 0, TF24_COL_MAJOR = 1 } tf24_layout;
+
+typedef enum {
+  TF24_PRUNE_MAGNITUDE = 0, /* keep the 2 largest |x| per group, ties -> larger index */
+  TF24_PRUNE_MASK = 1,      /* keep what a supplied mask says */
+  TF24_PRUNE_MVUE = 2       /* MVUE24 sampling from a supplied U(0,1) tensor */
+} tf24_prune_mode;
+
+typedef enum { TF24_ACT_NONE = 0, TF24_ACT_RELU = 1, TF24_ACT_SILU = 2 } tf24_activation;
+
+/* Library version string, e.g. "tf24 0.1.0 gfx950". Host only. */
+const char* tf24_version(void);
+
+/* Message of the last failing call on this thread ("" if none). Host only. */
+const char* tf24_last_error(void);
+
+/*
+ * Dense -> 2:4 prune + compress.
+ * Replaces sparse_semi_structured_from_dense_triton and its two Triton kernels
+ * (sparse/_semi_structured_conversions.py:431-661, :664-1069, launcher :1072-1132),
+ * called from SparseSemiStructuredTensor.__init__ (sparse/semi_structured.py:244-245).
+ *   dense      [m,k] in_dtype (F32|F16|BF16), (layout, ld)
+ *   mode       MAGNITUDE | MASK (mask required) | MVUE (rand required)
+ *   mask       [m,k] mask_dtype (U8|F16|BF16|F32), nonzero = kept, same layout, leading dim mask_ld
+ *   rand       [m,k] F32 uniforms in [0,1), same layout, leading dim rand_ld; group g of row r
+ *              uses rand[r,4g] and rand[r,4g+1]
+ *   values     [m,k/2] out_dtype (F16|BF16|E4M3), row-major contiguous
+ *   meta       canonical int16 [m,k/16] (F16|BF16) or int32 [m,k/32] (E4M3), row-major contiguous
+ * Shape rules (sparse/semi_structured.py:24-30,188-200): m % 32 == 0, k % 64 == 0 for 16-bit
+ * values, k % 128 == 0 for 8-bit values.
+ */
+int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                        int mode, const void* mask, int mask_dtype, int64_t mask_ld,
+                        const float* rand, int64_t rand_ld,
+                        void* values, int out_dtype, void* meta, void* stream);
+
+/* The argument checks of tf24_prune_compress without touching the GPU (pointers are only
+ * tested for NULL-ness through the has_* flags). Host only. */
+int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld, int64_t m, int64_t k, int mode,
+                                 int has_mask, int mask_dtype, int64_t mask_ld, int has_rand, int64_t rand_ld,
+                                 int out_dtype);
+
+/*
+ * Compressed -> dense.  Replaces _sparse_semi_structured_to_dense_kernel
+ * (sparse/_semi_structured_conversions.py:1163-1274) used by SparseSemiStructuredTensor.to_dense
+ * (sparse/semi_structured.py:554-572).  values [m,k/2] dtype, meta canonical, dense_out [m,k]
+ * row-major contiguous of the same dtype.
+ */
+int tf24_decompress(const void* values, int dtype, const void* meta, int64_t m, int64_t k,
+                    void* dense_out, void* stream);
+
+/*
+ * Transposable 4x4 mask search over the 90 row-and-column 2:4 patterns.
+ * Replaces _to_transposable_sparse_semi_structured_kernel and its launcher
+ * (sparse/transposable_semi_structured.py:8-47, :50-94) behind TransposableSparse.forward (:198-200).
+ *   dense [m,k] dtype (F32|F16|BF16), (layout, ld); m % 32 == 0, k % 64 == 0
+ *   sparse_out (may be NULL) dense*mask, same dtype/layout/ld;  mask_out bytes (0/1), same layout/ld
+ */
+int tf24_transposable_mask(const void* dense, int dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                           int use_abs, void* sparse_out, uint8_t* mask_out, void* stream);
+int tf24_transposable_mask_validate(int dtype, int layout, int64_t ld, int64_t m, int64_t k);
+
+/*
+ * Dense-shaped 2:4 operators: outputs have the dense dtype/layout/ld and are written completely
+ * (zeros at dropped positions).  k % 4 == 0 (row-major: k % 8 == 0 for 16-bit types).
+ *   tf24_soft_threshold24  S-STE soft threshold, replaces _soft_threshold24_triton
+ *                          (sparse/triton_ops.py:157-227, math sparse/utils.py:72-90)
+ *   tf24_sparse24_dense    magnitude pruning, replaces _sparse24_triton (sparse/triton_ops.py:84-154)
+ *   tf24_mvue24_dense      MVUE24 with supplied uniforms, replaces _MVUE24_approx_triton
+ *                          (sparse/triton_ops.py:10-81); mask_out unused (pass NULL)
+ */
+int tf24_soft_threshold24(const void* dense, int dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                          void* sparse_out, void* mask_out, void* stream);
+int tf24_sparse24_dense(const void* dense, int dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                        void* sparse_out, void* mask_out, void* stream);
+int tf24_mvue24_dense(const void* dense, int dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                      const float* rand, int64_t rand_ld, void* sparse_out, void* stream);
+
+/*
+ * Masked decay, in place: grad[i] += alpha * p[i] where mask[i] == 0.
+ * Replaces masked_add_kernel / masked_add_ (sparse/decay.py:7-37).  Flat over n elements
+ * (the reference requires identical strides and indexes storage linearly).
+ *   grad F32|F16|BF16, p F32|F16|BF16, mask U8|F32|F16|BF16
+ */
+int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, const void* mask, int mask_dtype,
+                    int64_t n, float alpha, void* stream);
+
+/*
+ * 2:4 sparse x dense matmul on SMFMAC, float32 accumulation:
+ *     C[i,j] = act( sum_k A[i,k] * B(k,j) + bias ),   A sparse [n_sparse, k], compressed.
+ * Replaces sparse.cutlass.my_sparse_semi_structured_linear
+ * (sparse/csrc/mySparseSemiStructuredLinear_cuda.cu:498-817, CUTLASS SparseGemm :61-76),
+ * bound at sparse/sparse_semi_structured_linear.py:4-5.
+ *   a_values [n_sparse,k/2], a_meta canonical; dtype F16|BF16|E4M3 (B has the same dtype)
+ *   b          dense operand, n_dense "columns" j: b_layout TF24_ROW_MAJOR means B is stored
+ *              [n_dense, k] (k contiguous, element (k,j) at j*ldb + k: the X of X.W^T);
+ *              TF24_COL_MAJOR means stored [k, n_dense] (element (k,j) at k*ldb + j)
+ *   c          output; c_layout TF24_ROW_MAJOR stores C[i,j] at i*ldc + j ([n_sparse,n_dense]);
+ *              TF24_COL_MAJOR stores it at j*ldc + i ([n_dense,n_sparse]: the Y of X.W^T)
+ *   bias       NULL or [n_sparse] of out_dtype's float family (added per sparse row i)
+ *   scale      multiplies the accumulator before bias (1.0 for 16-bit; scale_a*scale_b for fp8)
+ * Shape rules (.cu:101-109): n_sparse % 32 == 0, k % 64 == 0 (16-bit) / 128 (8-bit),
+ * n_dense % 8 == 0 (16-bit) / 16 (8-bit).
+ */
+int tf24_spmm(const void* a_values, const void* a_meta, int dtype, int64_t n_sparse, int64_t k,
+              const void* b, int b_layout, int64_t ldb, int64_t n_dense,
+              void* c, int out_dtype, int c_layout, int64_t ldc,
+              const void* bias, float scale, int activation, void* stream);
+int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_layout, int64_t ldb, int64_t n_dense,
+                       int out_dtype, int c_layout, int64_t ldc, int activation);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TF24_H */

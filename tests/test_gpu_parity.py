@@ -1,0 +1,325 @@
+"""GPU parity: every HIP kernel, called through the Python API -> ctypes -> C ABI, against the CPU
+oracle on the same seeded inputs.  Bit-exact for masks, metadata, compressed values and the
+element-wise operators; stated tolerances for the matmul."""
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+F16, BF16, F32, E4M3 = torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn
+
+
+def bits(t):
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.bool:
+        return t
+    return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32}[t.element_size()])
+
+
+def assert_same(got, want, what=""):
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    assert got.dtype == want.dtype, (what, got.dtype, want.dtype)
+    g, w = bits(got), bits(want)
+    if not g.equal(w):
+        bad = (g != w).nonzero()
+        raise AssertionError(f"{what}: {bad.shape[0]} of {g.numel()} elements differ, first at {bad[0].tolist()}: "
+                             f"got {got.detach().cpu()[tuple(bad[0])]} want {want[tuple(bad[0])]}")
+
+
+def randn(shape, dtype, seed, scale=1.0, ties=False):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g) * scale
+    if ties:   # coarse grid: many equal magnitudes inside groups
+        x = torch.round(x * 2) / 2
+    return x.to(dtype)
+
+
+def maybe_t(x, col_major):
+    """A logical tensor equal to x, stored column-major when asked (like W.T of a row-major W)."""
+    return x.t().contiguous().t() if col_major else x
+
+
+# ------------------------------------------------------------------ prune + compress
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("in_dtype", [F16, BF16, F32])
+@pytest.mark.parametrize("out_dtype", [F16, BF16, E4M3])
+@pytest.mark.parametrize("shape", [(32, 128), (96, 320 + 64), (64, 1024)])
+def test_magnitude_compress(cuda, shape, in_dtype, out_dtype, col_major):
+    import sparse
+    w = randn(shape, in_dtype, 11, ties=(shape[0] == 96))
+    want_v, want_m = oracle.compress24(w, out_dtype=out_dtype)
+    s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major), dtype=out_dtype)
+    assert s.shape == w.shape and s.dtype == out_dtype
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+    assert_same(s.to_dense(), oracle.decompress24(want_v, want_m), "to_dense")
+
+
+def test_docstring_known_answer(cuda):
+    import sparse
+    a = torch.tensor([0.0, 0.0, 1.0, 1.0]).tile((128, 32)).half().to(cuda)
+    s = sparse.to_sparse_semi_structured(a)
+    assert s.values().eq(1).all() and s.values().shape == (128, 64)
+    assert s.indices().eq(-4370).all() and s.indices().dtype == torch.int16
+    assert s.indices_cutlass().eq(-4370).all()
+
+
+def test_config1_compress_and_mm(cuda):
+    """BASELINE config 1 (the reference's CPU-runnable case), on the GPU path."""
+    import sparse
+    g = torch.Generator().manual_seed(0)
+    w = (0.02 * torch.randn(3072, 768, generator=g)).half()
+    x = torch.randn(12288, 768, generator=g)
+    want_v, want_m = oracle.compress24(w)
+    s = sparse.to_sparse_semi_structured(w.to(cuda))
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+    mask = oracle.prune24_mask(w)
+    ref = oracle.spmm_ref(x.half(), torch.where(mask, w, torch.zeros_like(w)))
+    out = torch.mm(x.half().to(cuda), s.t()).float().cpu()
+    rel = (out - ref).norm() / ref.norm()
+    assert out.shape == (12288, 3072) and rel < 1e-2, rel
+
+
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("mask_dtype", [torch.bool, F16, F32])
+@pytest.mark.parametrize("in_dtype,out_dtype", [(F32, F16), (F16, F16), (BF16, BF16), (F32, E4M3)])
+def test_mask_compress(cuda, in_dtype, out_dtype, mask_dtype, col_major):
+    import sparse
+    w = randn((64, 256), in_dtype, 12)
+    _, mask = oracle.transposable_mask(w.float())
+    g = torch.Generator().manual_seed(13)
+    mask[:8] = torch.rand(8, 256, generator=g) < 0.5            # invalid groups follow the truth table
+    mask = mask.to(mask_dtype)
+    want_v, want_m = oracle.compress24(w, mask=mask, out_dtype=out_dtype)
+    s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major), mask=maybe_t(mask.to(cuda), col_major), dtype=out_dtype)
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+
+
+def test_mask_layout_mismatch_is_copied(cuda):
+    import sparse
+    w = randn((64, 128), F16, 14)
+    mask = oracle.prune24_mask(w)
+    want_v, want_m = oracle.compress24(w, mask=mask)
+    # column-major dense with a row-major mask and vice versa
+    s1 = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), True), mask=mask.to(cuda))
+    s2 = sparse.to_sparse_semi_structured(w.to(cuda), mask=maybe_t(mask.to(cuda), True))
+    for s in (s1, s2):
+        assert_same(s.values(), want_v)
+        assert_same(s.indices(), want_m)
+
+
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("in_dtype,out_dtype", [(BF16, F16), (F16, F16), (F32, BF16), (BF16, E4M3), (F32, E4M3)])
+@pytest.mark.parametrize("shape", [(32, 128), (128, 640)])
+def test_mvue_compress(cuda, shape, in_dtype, out_dtype, col_major):
+    import sparse
+    w = randn(shape, in_dtype, 15)
+    w[0, :8] = 0                                                 # degenerate all-zero groups
+    u = torch.rand(shape, generator=torch.Generator().manual_seed(16))
+    u[1, 1] = 0.0                                                # r1 == 0: a single element may be kept
+    want_v, want_m, _ = oracle.mvue24(w, u, out_dtype=out_dtype)
+    s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major), MVUE24=True, rand=maybe_t(u.to(cuda), col_major), dtype=out_dtype)
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+
+
+def test_mvue_default_rand_keeps_two(cuda):
+    import sparse
+    w = randn((64, 128), F16, 17).to(cuda)
+    torch.manual_seed(0)
+    s = sparse.to_sparse_semi_structured(w, MVUE24=True)
+    dense = s.to_dense()
+    assert (dense != 0).reshape(-1, 4).sum(-1).le(2).all()
+
+
+def test_compress_errors(cuda):
+    import sparse
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(torch.zeros(32, 64, dtype=F16))                       # not on the GPU
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(torch.zeros(2, 32, 64, dtype=F16, device=cuda))       # not 2-d
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(torch.zeros(32, 64, dtype=F16, device=cuda), dtype=torch.float64)
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(torch.zeros(48, 64, dtype=F16, device=cuda))
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(torch.zeros(32, 64, dtype=F16, device=cuda), dtype=E4M3)  # needs k % 128
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(torch.zeros(32, 64, dtype=F16, device=cuda), MVUE24=True,
+                                         mask=torch.ones(32, 64, dtype=torch.bool, device=cuda))
+
+
+# ------------------------------------------------------------------ transposable search
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("use_abs", [True, False])
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+@pytest.mark.parametrize("ties", [False, True])
+def test_transposable(cuda, dtype, use_abs, col_major, ties):
+    import sparse
+    w = randn((96, 192), dtype, 21, ties=ties)
+    if ties:
+        w[:4, :8] = 0
+        w[4:8, :4] = 1
+    want_s, want_m = oracle.transposable_mask(w, use_abs=use_abs)
+    got_s, got_m = sparse.TransposableSparse(abs=use_abs)(maybe_t(w.to(cuda), col_major))
+    assert got_m.dtype == torch.bool
+    assert_same(got_m, want_m, "mask")
+    assert_same(got_s, want_s, "sparse")
+    if ties or dtype != F32:
+        _, brute, _ = oracle.transposable_mask_bruteforce(w, use_abs=use_abs)
+        if ties:
+            assert_same(got_m, brute, "mask vs 90-way brute force")
+
+
+def test_transposable_errors(cuda):
+    import sparse
+    ts = sparse.TransposableSparse()
+    for shape in [(33, 64), (32, 32)]:
+        with pytest.raises(RuntimeError):
+            ts(torch.zeros(shape, device=cuda))
+    with pytest.raises(RuntimeError):
+        ts(torch.zeros(32, 64, dtype=torch.float64, device=cuda))
+    with pytest.raises(RuntimeError):
+        ts(torch.zeros(2, 32, 64, device=cuda))
+
+
+# ------------------------------------------------------------------ dense-shaped operators
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_soft_threshold(cuda, dtype, col_major):
+    import sparse
+    w = randn((64, 256), dtype, 31, ties=(dtype == F16))
+    want_s, want_m = oracle.soft_threshold24(w)
+    got_s, got_m = sparse.soft_threshold24_triton(maybe_t(w.to(cuda), col_major))
+    assert_same(got_s, want_s, "sparse")
+    assert_same(got_m, want_m, "mask")
+    assert got_s.stride() == maybe_t(w, col_major).stride()
+
+
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_sparse24_and_mvue_dense(cuda, dtype, col_major):
+    import sparse
+    w = randn((64, 256), dtype, 32)
+    want_s, want_m = oracle.sparse24_dense(w)
+    got_s, got_m = sparse.sparse24_triton(maybe_t(w.to(cuda), col_major))
+    assert_same(got_s, want_s, "sparse24")
+    assert_same(got_m, want_m, "mask24")
+    u = torch.rand(w.shape, generator=torch.Generator().manual_seed(33))
+    got = sparse.MVUE24_approx_triton(maybe_t(w.to(cuda), col_major), rand=maybe_t(u.to(cuda), col_major))
+    assert_same(got, oracle.mvue24_dense(w, u), "mvue dense")
+
+
+# ------------------------------------------------------------------ masked decay
+@pytest.mark.parametrize("gdt,pdt,mdt", [(F32, F32, torch.bool), (F32, BF16, torch.bool), (F32, F32, F32),
+                                         (BF16, BF16, BF16), (F16, F32, torch.uint8)])
+@pytest.mark.parametrize("n", [(64, 64), (7, 13), (1000003,)])
+def test_masked_add(cuda, gdt, pdt, mdt, n):
+    import sparse
+    g = torch.Generator().manual_seed(41)
+    grad = (1e-3 * torch.randn(n, generator=g)).to(gdt)
+    p = torch.randn(n, generator=g).to(pdt)
+    mask = (torch.rand(n, generator=g) < 0.5).to(mdt)
+    want = oracle.masked_add(grad, p, mask, alpha=2e-4)
+    gg = grad.to(cuda)
+    assert sparse.masked_add_(gg, p.to(cuda), mask.to(cuda), alpha=2e-4) is None
+    assert_same(gg, want)
+
+
+def test_masked_add_reference_vector(cuda):
+    import sparse
+    grad = torch.tensor([1.0, 1.0, 1.0, 1.0], device=cuda)
+    sparse.masked_add_(grad, torch.tensor([1.0, 2.0, 3.0, 4.0], device=cuda), torch.tensor([1.0, 0.0, 1.0, 0.0], device=cuda), alpha=0.03)
+    assert torch.allclose(grad.cpu(), torch.tensor([1.0, 1.06, 1.0, 1.12]), atol=1e-7)
+
+
+# ------------------------------------------------------------------ 2:4 matmul
+def _small_ints(shape, seed, lo=-3, hi=4):
+    return torch.randint(lo, hi, shape, generator=torch.Generator().manual_seed(seed)).float()
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, E4M3])
+@pytest.mark.parametrize("dims", [(32, 128, 16), (64, 256, 40), (96, 384, 200), (160, 1024, 72)])
+def test_spmm_exact_small_integers(cuda, dtype, dims):
+    """Small-integer operands: every product and partial sum is exact in float32, so the
+    result must EQUAL the dense masked product -- pins operand and index layout."""
+    import sparse
+    n, k, m = dims
+    if dtype == E4M3 and m % 16:
+        m += 8
+    w = _small_ints((n, k), 51).to(dtype)
+    x = _small_ints((m, k), 52).to(dtype)
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    out = torch.mm(x.to(cuda), s.t())                      # second operand sparse: x . W^T
+    assert out.shape == (m, n)
+    assert out.dtype == (torch.float32 if dtype == E4M3 else dtype)
+    assert out.float().cpu().equal(ref)
+    # first operand sparse: W . B with B [k, j] row-major (k strided) and as a transposed view
+    b = x.t().contiguous()
+    out2 = torch.mm(s, b.to(cuda))
+    assert out2.shape == (n, m) and out2.float().cpu().equal(ref.t())
+    out3 = torch.mm(s, x.to(cuda).t())
+    assert out3.float().cpu().equal(ref.t())
+    # second operand sparse with a column-major x
+    out4 = torch.mm(maybe_t(x.to(cuda), True), s.t())
+    assert out4.float().cpu().equal(ref)
+
+
+@pytest.mark.parametrize("dtype,tol", [(F16, 1e-2), (BF16, 1e-2), (E4M3, 5e-2)])
+def test_spmm_random_tolerance(cuda, dtype, tol):
+    import sparse
+    n, k, m = 256, 512, 328 if dtype != E4M3 else 336
+    w = randn((n, k), F32, 53, scale=0.02)
+    x = randn((m, k), F32, 54)
+    if dtype == E4M3:
+        sw, sx = 448.0 / w.abs().max(), 448.0 / x.abs().max()
+        wq, xq = (w * sw).to(dtype), (x * sx).to(dtype)
+    else:
+        sw = sx = 1.0
+        wq, xq = w.to(dtype), x.to(dtype)
+    mask = oracle.prune24_mask(wq.float())
+    ref = oracle.spmm_ref(xq.float(), torch.where(mask, wq.float(), torch.zeros(())))
+    s = sparse.to_sparse_semi_structured(wq.to(cuda), dtype=dtype)
+    out = torch.mm(xq.to(cuda), s.t()).float().cpu()
+    rel = (out - ref).norm() / ref.norm()
+    assert rel < tol, rel
+
+
+def test_spmm_bias_linear_padding(cuda):
+    import sparse
+    n, k, m = 64, 128, 21                                   # m is padded to 24 and sliced back
+    w = _small_ints((n, k), 55).half()
+    x = _small_ints((3, 7, k), 56).half()
+    bias = _small_ints((n,), 57).half()
+    mask = oracle.prune24_mask(w)
+    wm = torch.where(mask, w, torch.zeros_like(w))
+    s = sparse.to_sparse_semi_structured(w.to(cuda))
+    ref = oracle.linear_ref(x, wm, bias)
+    out = torch.nn.functional.linear(x.to(cuda), s, bias.to(cuda))
+    assert out.shape == (3, 7, n) and out.float().cpu().equal(ref)
+    out = torch.addmm(bias.to(cuda), x.reshape(m, k).to(cuda), s.t())
+    assert out.float().cpu().equal(ref.reshape(m, n))
+    with torch.inference_mode():
+        out = torch.nn.functional.linear(x.to(cuda), s, bias.to(cuda))
+    assert out.float().cpu().equal(ref)
+
+
+def test_dispatch_rules(cuda):
+    import sparse
+    w = _small_ints((32, 64), 58).half().to(cuda)
+    s = sparse.to_sparse_semi_structured(w)
+    assert s.t().transposed and s.t().shape == (64, 32) and not s.t().t().transposed
+    assert s.detach().values().data_ptr() == s.values().data_ptr()
+    x = torch.ones(8, 64, dtype=F16, device=cuda)
+    with pytest.raises(NotImplementedError):
+        torch.mm(x, s)                                     # second operand must be transposed
+    with pytest.raises(NotImplementedError):
+        torch.mm(s.t(), x.t())                             # first operand must not be
+    with pytest.raises(NotImplementedError):
+        s + 1
