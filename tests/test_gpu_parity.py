@@ -255,10 +255,11 @@ def test_spmm_exact_small_integers(cuda, dtype, dims):
     x = _small_ints((m, k), 52).to(dtype)
     mask = oracle.prune24_mask(w.float())
     ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
-    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
     out = torch.mm(x.to(cuda), s.t())                      # second operand sparse: x . W^T
     assert out.shape == (m, n)
     assert out.dtype == (torch.float32 if dtype == E4M3 else dtype)
+    ref = ref.to(out.dtype).float()                        # the kernel rounds the exact sum once
     assert out.float().cpu().equal(ref)
     # first operand sparse: W . B with B [k, j] row-major (k strided) and as a transposed view
     b = x.t().contiguous()
@@ -285,7 +286,7 @@ def test_spmm_random_tolerance(cuda, dtype, tol):
         wq, xq = w.to(dtype), x.to(dtype)
     mask = oracle.prune24_mask(wq.float())
     ref = oracle.spmm_ref(xq.float(), torch.where(mask, wq.float(), torch.zeros(())))
-    s = sparse.to_sparse_semi_structured(wq.to(cuda), dtype=dtype)
+    s = sparse.to_sparse_semi_structured(wq.float().to(cuda), dtype=dtype)
     out = torch.mm(xq.to(cuda), s.t()).float().cpu()
     rel = (out - ref).norm() / ref.norm()
     assert rel < tol, rel
