@@ -351,6 +351,203 @@ spmm_tiled(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_m
     }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Pipelined kernel: same tiling as spmm_tiled, but operands go global -> LDS directly
+// (GLOBAL_LOAD_LDS_DWORDX4: lane l of a wave writes LDS[base + 16*l], so a wave fills 1 KB of
+// contiguous LDS) through a ring of three stage buffers: while stage s is multiplied, the loads
+// of stages s+1 and s+2 are in flight, which covers the L2/HBM latency that one stage of math
+// cannot.  LDS rows are unpadded; bank conflicts are avoided by XOR-swizzling the 16-byte chunk
+// index with row bits (B: chunk ^ ((row>>1)&7) in 128-byte rows, A: chunk ^ ((row>>2)&3) in
+// 64-byte rows), applied on the global side of the copy and again in the fragment reads.
+// The three buffers are separate LDS objects and the stage loop is unrolled by three, so that
+// every LDS access names its buffer statically.
+// ------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// The copies are issued from inline assembly so that the compiler's wait-count insertion does not
+// see them: it would otherwise drain all outstanding copies (vmcnt(0)) before every LDS read, because
+// it cannot tell the three stage buffers apart.  Ordering is enforced by hand with s_waitcnt vmcnt(N)
+// before the stage barrier.  M0 carries the wave-uniform LDS base of the copy.
+__device__ __forceinline__ uint32_t lds_offset(const void* p) {
+  return (uint32_t)(uintptr_t)(lds_ptr_t)p;
+}
+__device__ __forceinline__ void g2l16(const uint8_t* g, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void g2l4(const uint8_t* g, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
+}
+
+template <typename T, typename OutT, bool C_JMAJOR>
+__global__ void __launch_bounds__(TileCfg::THREADS)
+spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
+          const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
+          OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act,
+          int tiles_i, int tiles_j) {
+  using C = TileCfg;
+  constexpr int ES = sizeof(T);
+  constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
+  constexpr int M_STEP = M_ROW / C::STEPS;
+  constexpr int A_STAGE = C::BI * C::A_ROW, B_STAGE = C::BJ * C::B_ROW, M_STAGE = C::BI * M_ROW;
+  __shared__ __attribute__((aligned(1024))) uint8_t s_a0[A_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_a1[A_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_a2[A_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b0[B_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b1[B_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_b2[B_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_m0[M_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_m1[M_STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t s_m2[M_STAGE];
+
+  const int ntiles = tiles_i * tiles_j;
+  const int per_xcd = (ntiles + 7) / 8;
+  const int bid = blockIdx.x;
+  const int tile = (bid & 7) * per_xcd + (bid >> 3);
+  if (tile >= ntiles) return;
+  constexpr int GH = 4;
+  const int group = tile / (GH * tiles_j);
+  const int gh = min(GH, tiles_i - group * GH);
+  const int in_group = tile - group * GH * tiles_j;
+  const int tile_i = group * GH + in_group % gh;
+  const int tile_j = in_group / gh;
+  const int64_t i0 = (int64_t)tile_i * C::BI, j0 = (int64_t)tile_j * C::BJ;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wi = wave >> 2, wj = wave & 3;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const int64_t a_pitch = (k / 2) * ES;
+  const int64_t m_pitch = k / 8;
+  const int nstages = (int)((k * ES) / C::KB);
+
+  // ---- per-lane global sources of the copies (stage 0), LDS destinations are wave-uniform
+  const uint8_t* gb[4];
+  const uint8_t* ga[2];
+  const uint8_t* gm;
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const int row = (wave * 4 + q) * 8 + (lane >> 3);
+    const int ch = (lane & 7) ^ ((row >> 1) & 7);
+    gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16;
+  }
+#pragma unroll
+  for (int q = 0; q < 2; q++) {
+    const int row = (wave * 2 + q) * 16 + (lane >> 2);
+    const int ch = (lane & 3) ^ ((row >> 2) & 3);
+    ga[q] = a_values + min(i0 + row, n_sparse - 1) * a_pitch + ch * 16;
+  }
+  if constexpr (M_ROW == 8) {
+    const int row = wave * 32 + (lane >> 1);
+    gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch + (lane & 1) * 4;
+  } else {
+    const int row = (wave & 3) * 64 + lane;
+    gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch;
+  }
+  auto issue = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
+    const uint32_t la = lds_offset(sa), lb = lds_offset(sb), lm = lds_offset(sm);
+#pragma unroll
+    for (int q = 0; q < 4; q++) g2l16(gb[q] + (int64_t)st * C::B_ROW, lb + (wave * 4 + q) * 1024);
+#pragma unroll
+    for (int q = 0; q < 2; q++) g2l16(ga[q] + (int64_t)st * C::A_ROW, la + (wave * 2 + q) * 1024);
+    if constexpr (M_ROW == 8) g2l4(gm + (int64_t)st * M_ROW, lm + wave * 256);
+    else g2l16(gm + (int64_t)st * M_ROW, lm + (wave & 3) * 1024);    // waves 4-7 repeat the copy of waves 0-3
+  };
+  constexpr int LOADS_PER_STAGE = 7;   // copies per wave per stage
+
+  float16v acc[C::TI][C::TJ];
+#pragma unroll
+  for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+    for (int tj = 0; tj < C::TJ; tj++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[ti][tj][r] = 0.0f;
+
+  // ---- fragment offsets (swizzled)
+  const int a_row = wi * C::WI + l32, b_row = wj * C::WJ + l32;
+  const int a_sw = (l32 >> 2) & 3, b_sw = (l32 >> 1) & 7;
+  int a_off[C::STEPS], b_off[C::STEPS][2];
+#pragma unroll
+  for (int step = 0; step < C::STEPS; step++) {
+    a_off[step] = a_row * C::A_ROW + (((step * 2 + lh) ^ a_sw) * 16);
+#pragma unroll
+    for (int h = 0; h < 2; h++) b_off[step][h] = b_row * C::B_ROW + (((step * 4 + h * 2 + lh) ^ b_sw) * 16);
+  }
+  const int m_off = a_row * M_ROW + lh * (M_STEP / 2);
+
+  auto compute = [&](const uint8_t* sa, const uint8_t* sb, const uint8_t* sm) {
+#pragma unroll
+    for (int step = 0; step < C::STEPS; step++) {
+      int4v af[C::TI];
+      int idx[C::TI];
+      int8v bf[C::TJ];
+#pragma unroll
+      for (int ti = 0; ti < C::TI; ti++) {
+        af[ti] = *reinterpret_cast<const int4v*>(sa + a_off[step] + ti * 32 * C::A_ROW);
+        if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(sm + m_off + ti * 32 * M_ROW + step * M_STEP);
+        else idx[ti] = *reinterpret_cast<const int*>(sm + m_off + ti * 32 * M_ROW + step * M_STEP);
+      }
+#pragma unroll
+      for (int tj = 0; tj < C::TJ; tj++) {
+        const int4v lo = *reinterpret_cast<const int4v*>(sb + b_off[step][0] + tj * 32 * C::B_ROW);
+        const int4v hi = *reinterpret_cast<const int4v*>(sb + b_off[step][1] + tj * 32 * C::B_ROW);
+        bf[tj] = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+#pragma unroll
+      for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+        for (int tj = 0; tj < C::TJ; tj++) acc[ti][tj] = mma32<T>::run(af[ti], bf[tj], acc[ti][tj], idx[ti]);
+    }
+  };
+
+  // one pipeline step: stage `st` lives in (sa,sb,sm); the buffer freed by stage st-1 is (na,nb,nm)
+  auto pipe_step = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm, uint8_t* na, uint8_t* nb, uint8_t* nm) {
+    // loads of stage st were issued two steps ago; at most the loads of stage st+1 may still fly
+    // (a bare s_barrier: __syncthreads() would add a fence that drains every outstanding copy)
+    if (st + 1 < nstages) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (st + 2 < nstages) issue(st + 2, na, nb, nm);
+    compute(sa, sb, sm);
+  };
+
+  issue(0, s_a0, s_b0, s_m0);
+  if (nstages > 1) issue(1, s_a1, s_b1, s_m1);
+  int st = 0;
+  for (; st + 2 < nstages; st += 3) {
+    pipe_step(st, s_a0, s_b0, s_m0, s_a2, s_b2, s_m2);
+    pipe_step(st + 1, s_a1, s_b1, s_m1, s_a0, s_b0, s_m0);
+    pipe_step(st + 2, s_a2, s_b2, s_m2, s_a1, s_b1, s_m1);
+  }
+  if (st < nstages) { pipe_step(st, s_a0, s_b0, s_m0, s_a2, s_b2, s_m2); st++; }
+  if (st < nstages) { pipe_step(st, s_a1, s_b1, s_m1, s_a0, s_b0, s_m0); st++; }
+
+#pragma unroll
+  for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+    for (int tj = 0; tj < C::TJ; tj++) {
+      const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+        if (col >= n_dense || row >= n_sparse) continue;
+        OutT o[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          float v = acc[ti][tj][g * 4 + r] * scale;
+          if (bias) v += to_float(bias[row + r]);
+          o[r] = from_float<OutT>(apply_act(v, act));
+        }
+        if constexpr (C_JMAJOR) {
+          *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
+        }
+      }
+    }
+}
+
 template <typename T, typename OutT>
 int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
@@ -359,10 +556,10 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   const int per_xcd = (tiles_i * tiles_j + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
   if (c_layout == TF24_COL_MAJOR)
-    hipLaunchKernelGGL((spmm_tiled<T, OutT, true>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, true>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
                        (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
   else
-    hipLaunchKernelGGL((spmm_tiled<T, OutT, false>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, false>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
                        (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
   return check_launch("tf24_spmm");
 }
