@@ -445,14 +445,16 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     const int row = (wave & 3) * 64 + lane;
     gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch;
   }
+  // copy number q (0..6) of a stage: 4 x B, 2 x A, 1 x metadata
+  auto issue_one = [&](int q, int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
+    if (q < 4) g2l16(gb[q] + (int64_t)st * C::B_ROW, lds_offset(sb) + (wave * 4 + q) * 1024);
+    else if (q < 6) g2l16(ga[q - 4] + (int64_t)st * C::A_ROW, lds_offset(sa) + (wave * 2 + q - 4) * 1024);
+    else if constexpr (M_ROW == 8) g2l4(gm + (int64_t)st * M_ROW, lds_offset(sm) + wave * 256);
+    else g2l16(gm + (int64_t)st * M_ROW, lds_offset(sm) + (wave & 3) * 1024);    // waves 4-7 repeat the copy of waves 0-3
+  };
   auto issue = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
-    const uint32_t la = lds_offset(sa), lb = lds_offset(sb), lm = lds_offset(sm);
 #pragma unroll
-    for (int q = 0; q < 4; q++) g2l16(gb[q] + (int64_t)st * C::B_ROW, lb + (wave * 4 + q) * 1024);
-#pragma unroll
-    for (int q = 0; q < 2; q++) g2l16(ga[q] + (int64_t)st * C::A_ROW, la + (wave * 2 + q) * 1024);
-    if constexpr (M_ROW == 8) g2l4(gm + (int64_t)st * M_ROW, lm + wave * 256);
-    else g2l16(gm + (int64_t)st * M_ROW, lm + (wave & 3) * 1024);    // waves 4-7 repeat the copy of waves 0-3
+    for (int q = 0; q < 7; q++) issue_one(q, st, sa, sb, sm);
   };
   constexpr int LOADS_PER_STAGE = 7;   // copies per wave per stage
 
@@ -476,7 +478,11 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   }
   const int m_off = a_row * M_ROW + lh * (M_STEP / 2);
 
-  auto compute = [&](const uint8_t* sa, const uint8_t* sb, const uint8_t* sm) {
+  // Math of one stage.  The copies of the stage two ahead (into the buffer freed by the barrier) are
+  // issued one at a time between the matrix instructions: issued in a burst right after the barrier
+  // they would queue up in the texture-address unit and hold back every wave's fragment reads.
+  auto compute = [&](const uint8_t* sa, const uint8_t* sb, const uint8_t* sm, bool prefetch, int pst, uint8_t* na, uint8_t* nb,
+                     uint8_t* nm) {
 #pragma unroll
     for (int step = 0; step < C::STEPS; step++) {
       int4v af[C::TI];
@@ -495,9 +501,16 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
         bf[tj] = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
-      for (int ti = 0; ti < C::TI; ti++)
+      for (int ti = 0; ti < C::TI; ti++) {
 #pragma unroll
         for (int tj = 0; tj < C::TJ; tj++) acc[ti][tj] = mma32<T>::run(af[ti], bf[tj], acc[ti][tj], idx[ti]);
+        const int q = step * C::TI + ti;           // 8 slots per stage, 7 copies
+        if (q < 7 && prefetch) {
+          __builtin_amdgcn_sched_barrier(0);
+          issue_one(q, pst, na, nb, nm);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
     }
   };
 
@@ -507,8 +520,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     // (a bare s_barrier: __syncthreads() would add a fence that drains every outstanding copy)
     if (st + 1 < nstages) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE) : "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    if (st + 2 < nstages) issue(st + 2, na, nb, nm);
-    compute(sa, sb, sm);
+    compute(sa, sb, sm, st + 2 < nstages, st + 2, na, nb, nm);
   };
 
   issue(0, s_a0, s_b0, s_m0);
