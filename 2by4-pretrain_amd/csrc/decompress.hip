@@ -9,12 +9,19 @@ constexpr int kThreads = 256;
 
 template <typename T>
 __global__ void __launch_bounds__(kThreads)
-decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta, int64_t total_units, T* __restrict__ dense) {
-  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta, int64_t total_units, int64_t m, int64_t k,
+                  bool panel, T* __restrict__ dense) {
+  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;   // unit = 8 dense elements, row-major order
   if (u >= total_units) return;
+  int64_t src = u;
+  if (panel) {        // [k/KP][m][KP/8 units]
+    constexpr int UPP = (128 / (int)sizeof(T)) / 8;
+    const int64_t upr = k >> 3, row = u / upr, col8 = u - row * upr;
+    src = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
+  }
   Pack<T, 4> v;
-  v.load(values + u * 4);
-  const uint32_t mb = meta[u];
+  v.load(values + src * 4);
+  const uint32_t mb = meta[src];
   Pack<T, 8> out;
 #pragma unroll
   for (int i = 0; i < 8; i++) out.v[i] = T{};
@@ -32,27 +39,30 @@ decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta
 }
 
 template <typename T>
-int launch(const void* values, const void* meta, int64_t m, int64_t k, void* dense, hipStream_t s) {
+int launch(const void* values, const void* meta, bool panel, int64_t m, int64_t k, void* dense, hipStream_t s) {
   const int64_t total = m * (k / 8);
   dim3 grid((unsigned)((total + kThreads - 1) / kThreads));
-  hipLaunchKernelGGL((decompress_kernel<T>), grid, dim3(kThreads), 0, s, (const T*)values, (const uint8_t*)meta, total, (T*)dense);
+  hipLaunchKernelGGL((decompress_kernel<T>), grid, dim3(kThreads), 0, s, (const T*)values, (const uint8_t*)meta, total, m, k, panel, (T*)dense);
   return check_launch("tf24_decompress");
 }
 
 }  // namespace
 }  // namespace tf24
 
-extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, int64_t m, int64_t k,
+extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, int layout, int64_t m, int64_t k,
                                void* dense_out, void* stream) {
   using namespace tf24;
   const int64_t mult = dtype == TF24_E4M3 ? 32 : 16;
   if (m <= 0 || k <= 0 || k % mult) return fail(TF24_ERR_SHAPE, "tf24_decompress: k=%lld must be a positive multiple of %lld", (long long)k, (long long)mult);
   if (!values || !meta || !dense_out) return fail(TF24_ERR_ARG, "tf24_decompress: null pointer");
+  if (layout != TF24_COMPRESSED_CANONICAL && layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_decompress: bad compressed layout %d", layout);
+  const bool panel = layout == TF24_COMPRESSED_PANEL;
+  if (panel && k % (dtype == TF24_E4M3 ? 128 : 64)) return fail(TF24_ERR_SHAPE, "tf24_decompress: panel layout needs whole panels (k=%lld)", (long long)k);
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case TF24_F16: return launch<f16_t>(values, meta, m, k, dense_out, s);
-    case TF24_BF16: return launch<bf16_t>(values, meta, m, k, dense_out, s);
-    case TF24_E4M3: return launch<e4m3_t>(values, meta, m, k, dense_out, s);
+    case TF24_F16: return launch<f16_t>(values, meta, panel, m, k, dense_out, s);
+    case TF24_BF16: return launch<bf16_t>(values, meta, panel, m, k, dense_out, s);
+    case TF24_E4M3: return launch<e4m3_t>(values, meta, panel, m, k, dense_out, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_decompress: unsupported dtype %d", dtype);
 }

@@ -32,28 +32,45 @@ __device__ __forceinline__ uint32_t prune_group(const float (&x)[4], const MaskT
 }
 
 // ------------------------------------------------------------------ row-major
+// panel = false: canonical output, values [m, k/2] and metadata [m, k/8 bytes] row-major; units
+//   (8 dense elements) are walked along rows.
+// panel = true : panel output, [k/KP][m][64 bytes] values and [k/KP][m][KP/8 bytes] metadata with
+//   KP = 128 / sizeof(Out) dense elements per panel.  A block covers 32 rows x 256 dense columns:
+//   32 lanes read 256 consecutive columns of one row (full lines), the two half-waves take adjacent
+//   rows, so that every store instruction writes, per panel, the 2 x 64 contiguous bytes of a row pair.
 template <typename In, typename Out, int MODE, typename MaskT>
 __global__ void __launch_bounds__(kThreads)
 prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous) {
-  const int64_t upr = k >> 3;                 // 8-element units per row
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel) {
+  constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
+  const int64_t upr = k >> 3;                             // 8-element units per row
   const int64_t total = m * upr;
   const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
 #pragma unroll
   for (int it = 0; it < kUnroll; it++) {
     const int64_t u = base + (int64_t)it * kThreads;
-    const bool live = u < total;
+    bool live = u < total;
     uint32_t mbyte = 0;
     Pack<Out, 4> out;
-    int64_t row = 0, col8 = 0;
+    int64_t row = 0, col8 = 0, ounit = 0;
+    if (panel) {
+      row = (int64_t)blockIdx.x * 32 + it * 8 + (threadIdx.x >> 5);
+      col8 = (int64_t)blockIdx.y * 32 + (threadIdx.x & 31);
+      live = col8 < upr;                                   // m is a multiple of 32
+    }
     if (live) {
-      if (contiguous) {          // every leading dimension equals k: offsets are linear in u
-        col8 = u;
+      if (panel) {
+        ounit = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
       } else {
-        row = (int64_t)((uint32_t)u / (uint32_t)upr);
-        col8 = u - row * upr;
+        if (contiguous) {          // every leading dimension equals k: offsets are linear in u
+          col8 = u;
+        } else {
+          row = (int64_t)((uint32_t)u / (uint32_t)upr);
+          col8 = u - row * upr;
+        }
+        ounit = row * upr + col8;
       }
       Pack<In, 8> in;
       in.load(dense + row * ld + col8 * 8);
@@ -77,15 +94,14 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
         out.v[2 * g + 1] = from_float<Out>(select4(nib >> 2, y[0], y[1], y[2], y[3]));
         mbyte |= nib << (4 * g);
       }
-      out.store(values + row * (k >> 1) + col8 * 4);
+      out.store(values + ounit * 4);
     }
     // 4 adjacent lanes (32 dense columns of one row) -> one metadata dword
     uint32_t w = mbyte;
     w |= __shfl_down(mbyte, 1) << 8;
     w |= __shfl_down(mbyte, 2) << 16;
     w |= __shfl_down(mbyte, 3) << 24;
-    if (live && (threadIdx.x & 3) == 0)
-      *reinterpret_cast<uint32_t*>(meta + row * (k >> 3) + col8) = w;
+    if (live && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ounit) = w;
   }
 }
 
@@ -96,7 +112,7 @@ __global__ void __launch_bounds__(kThreads)
 prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta) {
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel) {
   constexpr int R = 16 / sizeof(In);
   constexpr int TR = 8 * R;          // tile rows
   constexpr int TC = 128;            // tile columns (32 groups)
@@ -144,10 +160,15 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     }
   }
   __syncthreads();
-  // values: TR rows x (TC/2)*sizeof(Out) bytes, 16 bytes per lane
+  // values: TR rows x (TC/2)*sizeof(Out) bytes, 16 bytes per lane.  Canonical output: row gr, byte
+  // offset (col0/2)*sizeof(Out) + seg*16 of a k/2-element row.  Panel output: the tile covers
+  // TC/KP panels (KP = 128/sizeof(Out) dense columns, 64 bytes of values per row); panel p of row gr
+  // lives at ((p*m + gr)*64) bytes.
   constexpr int VROW_BYTES = (TC / 2) * sizeof(Out);
   constexpr int LANES_PER_ROW = VROW_BYTES / 16;
   constexpr int ROWS_PER_PASS = kThreads / LANES_PER_ROW;
+  constexpr int KP = 128 / (int)sizeof(Out);
+  constexpr int MP = KP / 8;                             // metadata bytes per row per panel
   const int64_t vpitch_out = (k >> 1) * sizeof(Out);
 #pragma unroll
   for (int pass = 0; pass < (TR + ROWS_PER_PASS - 1) / ROWS_PER_PASS; pass++) {
@@ -159,7 +180,9 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       // LDS rows are padded by 4 bytes, so read as four dwords
       const uint32_t* sp = reinterpret_cast<const uint32_t*>(s_val + lr * VPITCH + seg * 16);
       uint4 v = make_uint4(sp[0], sp[1], sp[2], sp[3]);
-      *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(values) + gr * vpitch_out + gbyte) = v;
+      int64_t dst = gr * vpitch_out + gbyte;
+      if (panel) dst = ((gbyte >> 6) * m + gr) * 64 + (gbyte & 63);
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(values) + dst) = v;
     }
   }
   // metadata: TR rows x 16 bytes
@@ -168,45 +191,58 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     if (gr < m) {
       const uint32_t* sp = reinterpret_cast<const uint32_t*>(s_meta + tid * MPITCH);
       const int64_t mpitch_out = k >> 3;
-      uint8_t* dst = meta + gr * mpitch_out + (col0 >> 3);
-      // rows of the metadata matrix are only 8-byte aligned when k % 128 == 64
-      *reinterpret_cast<uint2*>(dst) = make_uint2(sp[0], sp[1]);
-      if (col0 + TC <= k) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(sp[2], sp[3]);
+      const bool full = col0 + TC <= k;                  // k % 128 == 64 leaves a half tile
+      if (!panel) {
+        uint8_t* dst = meta + gr * mpitch_out + (col0 >> 3);
+        // rows of the metadata matrix are only 8-byte aligned when k % 128 == 64
+        *reinterpret_cast<uint2*>(dst) = make_uint2(sp[0], sp[1]);
+        if (full) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(sp[2], sp[3]);
+      } else {
+        const int64_t mbyte0 = col0 >> 3;                // byte offset inside the row's canonical stream
+        uint8_t* dst = meta + ((mbyte0 / MP) * m + gr) * MP + (mbyte0 % MP);
+        *reinterpret_cast<uint2*>(dst) = make_uint2(sp[0], sp[1]);
+        if (full) {
+          const int64_t mbyte1 = mbyte0 + 8;
+          uint8_t* dst1 = meta + ((mbyte1 / MP) * m + gr) * MP + (mbyte1 % MP);
+          *reinterpret_cast<uint2*>(dst1) = make_uint2(sp[2], sp[3]);
+        }
+      }
     }
   }
 }
 
 template <typename In, typename Out, int MODE, typename MaskT>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
-           const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t stream) {
+           const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t stream) {
   if (layout == TF24_ROW_MAJOR) {
-    const int64_t total = m * (k >> 3);
-    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == k);
     const int64_t per_block = kThreads * kUnroll;
+    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == k);
+    const int64_t total = m * (k >> 3);
     dim3 grid((unsigned)((total + per_block - 1) / per_block));
+    if (panel) grid = dim3((unsigned)(m / 32), (unsigned)((k + 255) / 256));     // 32 rows x 256 columns per block
     hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
                        (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta,
-                       contiguous);
+                       contiguous, panel);
   } else {
     constexpr int R = 16 / sizeof(In);
     dim3 grid((unsigned)((k + 127) / 128), (unsigned)((m + 8 * R - 1) / (8 * R)));
     hipLaunchKernelGGL((prune_compress_col<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
-                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta);
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel);
   }
   return check_launch("tf24_prune_compress");
 }
 
 template <typename In, typename Out, int MODE>
 int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int mask_dtype,
-                  int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t s) {
+                  int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t s) {
   if constexpr (MODE != TF24_PRUNE_MASK) {
-    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, values, meta, s);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, values, meta, panel, s);
   } else {
     switch (mask_dtype) {
-      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
-      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
-      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
-      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, s);
+      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
+      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
+      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
+      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
     }
     return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported mask dtype %d", mask_dtype);
   }
@@ -214,25 +250,25 @@ int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t 
 
 template <typename In, typename Out>
 int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t s) {
+                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t s) {
   switch (mode) {
     case TF24_PRUNE_MAGNITUDE:
-      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
     case TF24_PRUNE_MASK:
-      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
     case TF24_PRUNE_MVUE:
-      return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
   }
   return fail(TF24_ERR_ARG, "tf24_prune_compress: bad mode %d", mode);
 }
 
 template <typename In>
 int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, hipStream_t s) {
+                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t s) {
   switch (out_dtype) {
-    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
-    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
-    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported output dtype %d", out_dtype);
 }
@@ -243,17 +279,20 @@ int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t
 extern "C" int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
                                    int mode, const void* mask, int mask_dtype, int64_t mask_ld,
                                    const float* rnd, int64_t rand_ld,
-                                   void* values, int out_dtype, void* meta, void* stream) {
+                                   void* values, int out_dtype, void* meta, int out_layout, void* stream) {
   using namespace tf24;
   int rc = tf24_prune_compress_validate(in_dtype, layout, ld, m, k, mode, mask != nullptr, mask_dtype, mask_ld,
                                         rnd != nullptr, rand_ld, out_dtype);
   if (rc != TF24_OK) return rc;
   if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "tf24_prune_compress: null dense/values/meta pointer");
+  if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
+    return fail(TF24_ERR_ARG, "tf24_prune_compress: bad compressed layout %d", out_layout);
+  const bool panel = out_layout == TF24_COMPRESSED_PANEL;
   hipStream_t s = (hipStream_t)stream;
   switch (in_dtype) {
-    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, s);
+    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported input dtype %d", in_dtype);
 }

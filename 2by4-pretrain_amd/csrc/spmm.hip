@@ -67,7 +67,7 @@ template <typename T, typename OutT, bool B_KCONTIG, bool C_JMAJOR>
 __global__ void __launch_bounds__(256)
 spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
              const T* __restrict__ b, int64_t ldb, int64_t n_dense,
-             OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
+             OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act, bool panel) {
   constexpr int KSTEP = mma16<T>::KSTEP;
   constexpr int ES = sizeof(T);                       // element size of values and B
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -89,9 +89,12 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 #pragma unroll
     for (int ti = 0; ti < 2; ti++) {
       const int64_t row = i0 + ti * 16 + li;
-      af[ti] = *reinterpret_cast<const int4v*>(a_values + row * a_pitch + (k0 / 2) * ES + lk * 16);
-      if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(a_meta + row * m_pitch + k0 / 8 + lk * 2);
-      else idx[ti] = *reinterpret_cast<const int*>(a_meta + row * m_pitch + k0 / 8 + lk * 4);
+      // one instruction step is exactly one panel (KSTEP dense columns: 64 value bytes, KSTEP/8 metadata bytes)
+      const int64_t voff = panel ? ((k0 / KSTEP) * n_sparse + row) * 64 : row * a_pitch + (k0 / 2) * ES;
+      const int64_t moff = panel ? ((k0 / KSTEP) * n_sparse + row) * (KSTEP / 8) : row * m_pitch + k0 / 8;
+      af[ti] = *reinterpret_cast<const int4v*>(a_values + voff + lk * 16);
+      if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(a_meta + moff + lk * 2);
+      else idx[ti] = *reinterpret_cast<const int*>(a_meta + moff + lk * 4);
     }
     int8v bf[2];
 #pragma unroll
@@ -147,14 +150,10 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 // ------------------------------------------------------------------------------------------
 // Tiled kernel (B with k contiguous): 512 lanes = 8 waves (2 along i x 4 along j) compute a
 // 256(i) x 256(j) tile; a wave owns 128 x 64 = 4 x 2 instructions of 32x32.  Operands are staged
-// through LDS in double-buffered stages of 128 bytes of dense k per row (two instruction steps);
-// the next stage's global loads are issued before the current stage's math and written to the
-// other LDS buffer after it, one barrier per stage.  Two waves per SIMD hide each other's LDS
-// and global latency.  Rows are padded by 16 bytes in LDS so that the 128-bit fragment reads
-// of 16 consecutive rows fall into distinct banks.
+// through LDS in stages of 128 bytes of dense k per row (two instruction steps).
 // Workgroup ids are remapped so that the 8 XCDs (ids are dealt round-robin) each walk a
-// contiguous range of tiles in a 4-tile-high grouped raster: concurrently resident tiles share
-// A rows and B columns in their XCD's L2.
+// contiguous range of tiles in an 8-tile-high grouped raster: the ~32 tiles resident on an XCD
+// form an 8 x 4 patch that shares A rows and B columns in that XCD's L2.
 // ------------------------------------------------------------------------------------------
 template <typename T> struct mma32;
 template <> struct mma32<f16_t> {
@@ -180,177 +179,10 @@ struct TileCfg {
   static constexpr int TI = WI / 32, TJ = WJ / 32;
   static constexpr int KB = 128;                 // bytes of dense k per row per stage
   static constexpr int STEPS = KB / 64;          // instruction steps per stage
-  static constexpr int A_ROW = KB / 2, A_PITCH = A_ROW + 16;
-  static constexpr int B_ROW = KB, B_PITCH = B_ROW + 16;
+  static constexpr int A_ROW = KB / 2;           // LDS bytes per row per stage: compressed values
+  static constexpr int B_ROW = KB;               //                              dense operand
+  static constexpr int GH = 8;                   // raster group height in tiles along i
 };
-
-template <typename T, typename OutT, bool C_JMAJOR>
-__global__ void __launch_bounds__(TileCfg::THREADS)
-spmm_tiled(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
-           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
-           OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act,
-           int tiles_i, int tiles_j) {
-  using C = TileCfg;
-  constexpr int ES = sizeof(T);
-  constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
-  constexpr int M_STEP = M_ROW / C::STEPS;                  // per instruction step (4 or 8)
-  constexpr int A_STAGE = C::BI * C::A_PITCH, B_STAGE = C::BJ * C::B_PITCH, M_STAGE = C::BI * M_ROW;
-  __shared__ __attribute__((aligned(16))) uint8_t s_a[2 * A_STAGE];
-  __shared__ __attribute__((aligned(16))) uint8_t s_b[2 * B_STAGE];
-  __shared__ __attribute__((aligned(16))) uint8_t s_m[2 * M_STAGE];
-
-  // ---- XCD-aware tile assignment
-  const int ntiles = tiles_i * tiles_j;
-  const int per_xcd = (ntiles + 7) / 8;
-  const int bid = blockIdx.x;
-  const int tile = (bid & 7) * per_xcd + (bid >> 3);
-  if (tile >= ntiles) return;
-  constexpr int GH = 4;                                     // group height in tiles along i
-  const int group = tile / (GH * tiles_j);
-  const int gh = min(GH, tiles_i - group * GH);
-  const int in_group = tile - group * GH * tiles_j;
-  const int tile_i = group * GH + in_group % gh;
-  const int tile_j = in_group / gh;
-  const int64_t i0 = (int64_t)tile_i * C::BI, j0 = (int64_t)tile_j * C::BJ;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wi = wave >> 2, wj = wave & 3;                  // 2 x 4 waves
-  const int l32 = lane & 31, lh = lane >> 5;
-
-  const int64_t a_pitch = (k / 2) * ES;                     // global bytes per row: values
-  const int64_t m_pitch = k / 8;                            //                      metadata
-  const int nstages = (int)((k * ES) / C::KB);
-
-  // ---- global -> register prefetch of one stage (A: 2 x 16 B, B: 4 x 16 B, meta: up to 16 B per thread)
-  int4v ra[2], rb[4];
-  int4v rm;
-  const uint8_t* ga[2];
-  const uint8_t* gb[4];
-  const uint8_t* gm;
-  int sa_off[2], sb_off[4], sm_off;
-#pragma unroll
-  for (int r = 0; r < 2; r++) {
-    const int cid = tid + r * C::THREADS;                   // 256 rows x 4 chunks
-    const int row = cid >> 2, ch = cid & 3;
-    const int64_t grow = min(i0 + row, n_sparse - 1);
-    ga[r] = a_values + grow * a_pitch + ch * 16;
-    sa_off[r] = row * C::A_PITCH + ch * 16;
-  }
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    const int cid = tid + r * C::THREADS;                   // 256 rows x 8 chunks
-    const int row = cid >> 3, ch = cid & 7;
-    const int64_t grow = min(j0 + row, n_dense - 1);
-    gb[r] = b + grow * ldb_bytes + ch * 16;
-    sb_off[r] = row * C::B_PITCH + ch * 16;
-  }
-  {
-    // metadata: one row per thread for the first 256 threads (M_ROW = 8) or 16 B per row (M_ROW = 16)
-    const int row = tid & 255;
-    const int64_t grow = min(i0 + row, n_sparse - 1);
-    gm = a_meta + grow * m_pitch;
-    sm_off = row * M_ROW;
-  }
-  auto load_stage = [&](int st) {
-#pragma unroll
-    for (int r = 0; r < 2; r++) ra[r] = *reinterpret_cast<const int4v*>(ga[r] + (int64_t)st * C::A_ROW);
-#pragma unroll
-    for (int r = 0; r < 4; r++) rb[r] = *reinterpret_cast<const int4v*>(gb[r] + (int64_t)st * C::B_ROW);
-    if (tid < 256) {
-      if constexpr (M_ROW == 8) {
-        const uint2 v = *reinterpret_cast<const uint2*>(gm + (int64_t)st * M_ROW);
-        rm[0] = v.x; rm[1] = v.y;
-      } else {
-        rm = *reinterpret_cast<const int4v*>(gm + (int64_t)st * M_ROW);
-      }
-    }
-  };
-  auto store_stage = [&](int buf) {
-#pragma unroll
-    for (int r = 0; r < 2; r++) *reinterpret_cast<int4v*>(s_a + buf * A_STAGE + sa_off[r]) = ra[r];
-#pragma unroll
-    for (int r = 0; r < 4; r++) *reinterpret_cast<int4v*>(s_b + buf * B_STAGE + sb_off[r]) = rb[r];
-    if (tid < 256) {
-      if constexpr (M_ROW == 8) *reinterpret_cast<uint2*>(s_m + buf * M_STAGE + sm_off) = make_uint2(rm[0], rm[1]);
-      else *reinterpret_cast<int4v*>(s_m + buf * M_STAGE + sm_off) = rm;
-    }
-  };
-
-  float16v acc[C::TI][C::TJ];
-#pragma unroll
-  for (int ti = 0; ti < C::TI; ti++)
-#pragma unroll
-    for (int tj = 0; tj < C::TJ; tj++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[ti][tj][r] = 0.0f;
-
-  // fragment read offsets inside a stage buffer
-  const int a_frag = (wi * C::WI + l32) * C::A_PITCH + lh * 16;       // + ti*32*A_PITCH + step*32
-  const int m_frag = (wi * C::WI + l32) * M_ROW + lh * (M_STEP / 2);  // + ti*32*M_ROW  + step*M_STEP
-  const int b_frag = (wj * C::WJ + l32) * C::B_PITCH + lh * 16;       // + tj*32*B_PITCH + step*64 (+32)
-
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
-  for (int st = 0; st < nstages; st++) {
-    const int buf = st & 1;
-    if (st + 1 < nstages) load_stage(st + 1);
-    const uint8_t* pa = s_a + buf * A_STAGE + a_frag;
-    const uint8_t* pm = s_m + buf * M_STAGE + m_frag;
-    const uint8_t* pb = s_b + buf * B_STAGE + b_frag;
-#pragma unroll
-    for (int step = 0; step < C::STEPS; step++) {
-      int4v af[C::TI];
-      int idx[C::TI];
-      int8v bf[C::TJ];
-#pragma unroll
-      for (int ti = 0; ti < C::TI; ti++) {
-        af[ti] = *reinterpret_cast<const int4v*>(pa + ti * 32 * C::A_PITCH + step * 32);
-        if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(pm + ti * 32 * M_ROW + step * M_STEP);
-        else idx[ti] = *reinterpret_cast<const int*>(pm + ti * 32 * M_ROW + step * M_STEP);
-      }
-#pragma unroll
-      for (int tj = 0; tj < C::TJ; tj++) {
-        const int4v lo = *reinterpret_cast<const int4v*>(pb + tj * 32 * C::B_PITCH + step * 64);
-        const int4v hi = *reinterpret_cast<const int4v*>(pb + tj * 32 * C::B_PITCH + step * 64 + 32);
-        bf[tj] = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int ti = 0; ti < C::TI; ti++)
-#pragma unroll
-        for (int tj = 0; tj < C::TJ; tj++) acc[ti][tj] = mma32<T>::run(af[ti], bf[tj], acc[ti][tj], idx[ti]);
-    }
-    if (st + 1 < nstages) store_stage(buf ^ 1);
-    __syncthreads();
-  }
-
-  // ---- epilogue: D layout column l%32, rows 8*(r/4) + 4*(l/32) + r%4
-#pragma unroll
-  for (int ti = 0; ti < C::TI; ti++)
-#pragma unroll
-    for (int tj = 0; tj < C::TJ; tj++) {
-      const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
-        if (col >= n_dense || row >= n_sparse) continue;
-        OutT o[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          float v = acc[ti][tj][g * 4 + r] * scale;
-          if (bias) v += to_float(bias[row + r]);
-          o[r] = from_float<OutT>(apply_act(v, act));
-        }
-        if constexpr (C_JMAJOR) {
-          *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
-        }
-      }
-    }
-}
-
 
 // ------------------------------------------------------------------------------------------
 // Pipelined kernel: same tiling as spmm_tiled, but operands go global -> LDS directly
@@ -379,7 +211,7 @@ __device__ __forceinline__ void g2l4(const uint8_t* g, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
 }
 
-template <typename T, typename OutT, bool C_JMAJOR>
+template <typename T, typename OutT, bool C_JMAJOR, bool PANEL>
 __global__ void __launch_bounds__(TileCfg::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
@@ -405,7 +237,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   const int bid = blockIdx.x;
   const int tile = (bid & 7) * per_xcd + (bid >> 3);
   if (tile >= ntiles) return;
-  constexpr int GH = 4;
+  constexpr int GH = C::GH;
   const int group = tile / (GH * tiles_j);
   const int gh = min(GH, tiles_i - group * GH);
   const int in_group = tile - group * GH * tiles_j;
@@ -432,31 +264,57 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     const int ch = (lane & 7) ^ ((row >> 1) & 7);
     gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16;
   }
+  // A and its metadata.  Canonical layout: rows strided by the row pitch, 64 value bytes (4 chunks)
+  // and M_ROW metadata bytes per row per stage.  Panel layout: stage st of rows i0..i0+255 is one
+  // contiguous run of 256*64 value bytes at (st*n_sparse + i0)*64 and 256*M_ROW metadata bytes.
+  int64_t a_stage_stride, m_stage_stride;
+  bool has_meta_copy = true;
+  if constexpr (PANEL) {
 #pragma unroll
-  for (int q = 0; q < 2; q++) {
-    const int row = (wave * 2 + q) * 16 + (lane >> 2);
-    const int ch = (lane & 3) ^ ((row >> 2) & 3);
-    ga[q] = a_values + min(i0 + row, n_sparse - 1) * a_pitch + ch * 16;
-  }
-  if constexpr (M_ROW == 8) {
-    const int row = wave * 32 + (lane >> 1);
-    gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch + (lane & 1) * 4;
+    for (int q = 0; q < 2; q++) {
+      const int row = (wave * 2 + q) * 16 + (lane >> 2);
+      const int ch = (lane & 3) ^ ((row >> 2) & 3);
+      ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16;
+    }
+    // metadata: 1 KB per copy = 128 rows (M_ROW 8) or 64 rows (M_ROW 16): waves 0..(2 or 4)-1
+    constexpr int M_COPIES = C::BI * M_ROW / 1024;
+    has_meta_copy = wave < M_COPIES;
+    const int row = (wave % M_COPIES) * (1024 / M_ROW) + lane * 16 / M_ROW;
+    // a 16-byte copy spans 16/M_ROW rows: clamp so that it never reaches past the last row
+    gm = a_meta + min(i0 + row, n_sparse - 16 / M_ROW) * M_ROW + (lane * 16) % M_ROW;
+    a_stage_stride = n_sparse * 64;
+    m_stage_stride = n_sparse * M_ROW;
   } else {
-    const int row = (wave & 3) * 64 + lane;
-    gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch;
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+      const int row = (wave * 2 + q) * 16 + (lane >> 2);
+      const int ch = (lane & 3) ^ ((row >> 2) & 3);
+      ga[q] = a_values + min(i0 + row, n_sparse - 1) * a_pitch + ch * 16;
+    }
+    if constexpr (M_ROW == 8) {
+      const int row = wave * 32 + (lane >> 1);
+      gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch + (lane & 1) * 4;
+    } else {
+      const int row = (wave & 3) * 64 + lane;
+      gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch;
+    }
+    a_stage_stride = C::A_ROW;
+    m_stage_stride = M_ROW;
   }
   // copy number q (0..6) of a stage: 4 x B, 2 x A, 1 x metadata
   auto issue_one = [&](int q, int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
     if (q < 4) g2l16(gb[q] + (int64_t)st * C::B_ROW, lds_offset(sb) + (wave * 4 + q) * 1024);
-    else if (q < 6) g2l16(ga[q - 4] + (int64_t)st * C::A_ROW, lds_offset(sa) + (wave * 2 + q - 4) * 1024);
-    else if constexpr (M_ROW == 8) g2l4(gm + (int64_t)st * M_ROW, lds_offset(sm) + wave * 256);
+    else if (q < 6) g2l16(ga[q - 4] + (int64_t)st * a_stage_stride, lds_offset(sa) + (wave * 2 + q - 4) * 1024);
+    else if constexpr (PANEL) {
+      if (has_meta_copy) g2l16(gm + (int64_t)st * m_stage_stride, lds_offset(sm) + wave * 1024);
+    } else if constexpr (M_ROW == 8) g2l4(gm + (int64_t)st * M_ROW, lds_offset(sm) + wave * 256);
     else g2l16(gm + (int64_t)st * M_ROW, lds_offset(sm) + (wave & 3) * 1024);    // waves 4-7 repeat the copy of waves 0-3
   };
   auto issue = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
 #pragma unroll
     for (int q = 0; q < 7; q++) issue_one(q, st, sa, sb, sm);
   };
-  constexpr int LOADS_PER_STAGE = 7;   // copies per wave per stage
+  constexpr int LOADS_PER_STAGE = 7;   // copies per wave per stage (6 for panel-layout waves without a metadata copy)
 
   float16v acc[C::TI][C::TJ];
 #pragma unroll
@@ -518,8 +376,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   auto pipe_step = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm, uint8_t* na, uint8_t* nb, uint8_t* nm) {
     // loads of stage st were issued two steps ago; at most the loads of stage st+1 may still fly
     // (a bare s_barrier: __syncthreads() would add a fence that drains every outstanding copy)
-    if (st + 1 < nstages) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (st + 1 >= nstages) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else if (has_meta_copy) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE - 1) : "memory");
     compute(sa, sb, sm, st + 2 < nstages, st + 2, na, nb, nm);
   };
 
@@ -561,29 +420,32 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 }
 
 template <typename T, typename OutT>
-int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
+int launch_tiled(const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
   using C = TileCfg;
   const int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI), tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
   const int per_xcd = (tiles_i * tiles_j + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
-  if (c_layout == TF24_COL_MAJOR)
-    hipLaunchKernelGGL((spmm_pipe<T, OutT, true>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
-                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
-  else
-    hipLaunchKernelGGL((spmm_pipe<T, OutT, false>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
-                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
+  const bool jm = c_layout == TF24_COL_MAJOR;
+#define TF24_GO(JM, PN)                                                                                                       \
+  hipLaunchKernelGGL((spmm_pipe<T, OutT, JM, PN>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, \
+                     (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j)
+  if (jm && panel) TF24_GO(true, true);
+  else if (jm) TF24_GO(true, false);
+  else if (panel) TF24_GO(false, true);
+  else TF24_GO(false, false);
+#undef TF24_GO
   return check_launch("tf24_spmm");
 }
 
 template <typename T, typename OutT>
-int launch_general(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
+int launch_general(const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                    int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
   dim3 grid((unsigned)((n_dense + 63) / 64), (unsigned)((n_sparse + 63) / 64));
   const bool kc = b_layout == TF24_ROW_MAJOR, jm = c_layout == TF24_COL_MAJOR;
 #define TF24_GO(KC, JM)                                                                                              \
   hipLaunchKernelGGL((spmm_general<T, OutT, KC, JM>), grid, dim3(256), 0, s, (const uint8_t*)av, (const uint8_t*)am, \
-                     n_sparse, k, (const T*)b, ldb, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act)
+                     n_sparse, k, (const T*)b, ldb, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, panel)
   if (kc && jm) TF24_GO(true, true);
   else if (kc) TF24_GO(true, false);
   else if (jm) TF24_GO(false, true);
@@ -593,20 +455,20 @@ int launch_general(const void* av, const void* am, int64_t n_sparse, int64_t k, 
 }
 
 template <typename T>
-int dispatch_out(int out_dtype, const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout,
+int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout,
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  hipStream_t s) {
   if (b_layout == TF24_ROW_MAJOR && n_sparse >= 64 && n_dense >= 64) {
     switch (out_dtype) {
-      case TF24_F16: return launch_tiled<T, f16_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-      case TF24_BF16: return launch_tiled<T, bf16_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-      case TF24_F32: return launch_tiled<T, float>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_F16: return launch_tiled<T, f16_t>(av, am, panel, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_BF16: return launch_tiled<T, bf16_t>(av, am, panel, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_F32: return launch_tiled<T, float>(av, am, panel, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
     }
   }
   switch (out_dtype) {
-    case TF24_F16: return launch_general<T, f16_t>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-    case TF24_BF16: return launch_general<T, bf16_t>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-    case TF24_F32: return launch_general<T, float>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_F16: return launch_general<T, f16_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_BF16: return launch_general<T, bf16_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_F32: return launch_general<T, float>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_spmm: unsupported output dtype %d", out_dtype);
 }
@@ -635,7 +497,7 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
   return TF24_OK;
 }
 
-extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int dtype, int64_t n_sparse, int64_t k,
+extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,
                          const void* b, int b_layout, int64_t ldb, int64_t n_dense,
                          void* c, int out_dtype, int c_layout, int64_t ldc,
                          const void* bias, float scale, int activation, void* stream) {
@@ -643,10 +505,12 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int dtype, in
   int rc = tf24_spmm_validate(dtype, n_sparse, k, b_layout, ldb, n_dense, out_dtype, c_layout, ldc, activation);
   if (rc) return rc;
   if (!a_values || !a_meta || !b || !c) return fail(TF24_ERR_ARG, "tf24_spmm: null pointer");
+  if (a_layout != TF24_COMPRESSED_CANONICAL && a_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_spmm: bad compressed layout %d", a_layout);
+  const bool panel = a_layout == TF24_COMPRESSED_PANEL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
-    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
   }
 }

@@ -16,6 +16,7 @@ F32, F16, BF16, E4M3, U8 = 0, 1, 2, 3, 4
 ROW_MAJOR, COL_MAJOR = 0, 1
 PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_SILU = 0, 1, 2
+COMPRESSED_CANONICAL, COMPRESSED_PANEL = 0, 1
 
 _DTYPES = {
     torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float8_e4m3fn: E4M3,
@@ -30,16 +31,16 @@ _f = ctypes.c_float
 _SIGNATURES = {
     "tf24_version": (ctypes.c_char_p, []),
     "tf24_last_error": (ctypes.c_char_p, []),
-    "tf24_prune_compress": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _p]),
+    "tf24_prune_compress": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p]),
     "tf24_prune_compress_validate": (_i, [_i, _i, _i64, _i64, _i64, _i, _i, _i, _i64, _i, _i64, _i]),
-    "tf24_decompress": (_i, [_p, _i, _p, _i64, _i64, _p, _p]),
+    "tf24_decompress": (_i, [_p, _i, _p, _i, _i64, _i64, _p, _p]),
     "tf24_transposable_mask": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _p, _p]),
     "tf24_transposable_mask_validate": (_i, [_i, _i, _i64, _i64, _i64]),
     "tf24_soft_threshold24": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _p, _p]),
     "tf24_sparse24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _p, _p]),
     "tf24_mvue24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _i64, _p, _p]),
     "tf24_masked_add": (_i, [_p, _i, _p, _i, _p, _i, _i64, _f, _p]),
-    "tf24_spmm": (_i, [_p, _p, _i, _i64, _i64, _p, _i, _i64, _i64, _p, _i, _i, _i64, _p, _f, _i, _p]),
+    "tf24_spmm": (_i, [_p, _p, _i, _i, _i64, _i64, _p, _i, _i64, _i64, _p, _i, _i, _i64, _p, _f, _i, _p]),
     "tf24_spmm_validate": (_i, [_i, _i64, _i64, _i, _i64, _i64, _i, _i, _i64, _i]),
 }
 

@@ -5,9 +5,12 @@ Mirrors the public surface of sparse/semi_structured.py of huyz2023/2by4-pretrai
 behaviour.  Differences, all deliberate:
   * one backend (hand-written HIP on SMFMAC); `_FORCE_CUTLASS` / `_FUSE_TRANSPOSE` are kept as
     inert attributes, `compressed_tensor_cusparselt` is always None;
-  * `meta_tensor_cutlass` holds the CANONICAL row-major nibble metadata (what one SMFMAC lane
-    consumes), not CUTLASS's reordered layout; `indices_cutlass()` exports the reordered form;
-  * compressed values are always row-major [m, k/2], also for column-major inputs (`W.T`);
+  * the compressed operand is STORED in the panel layout the SMFMAC matmul streams (tf24.h:
+    TF24_COMPRESSED_PANEL; class flag `_PANEL_LAYOUT`); `values()` / `indices()` /
+    `sparse_tensor_cutlass` / `meta_tensor_cutlass` materialise the canonical row-major form
+    (values [m, k/2], nibble metadata [m, k/16 | k/32]) on first use, also for column-major
+    inputs (`W.T`); the metadata is the canonical nibble stream, not CUTLASS's reordered layout --
+    `indices_cutlass()` exports the reordered form;
   * MVUE24 takes its uniforms from an optional `rand` tensor (drawn with torch.rand when omitted);
   * `addmm` / `linear` with a bias work (the reference passes a wrong keyword there).
 """
@@ -39,14 +42,27 @@ def _indices_dtype(values_dtype):
     raise RuntimeError(f"Datatype {values_dtype}  is not supported!")
 
 
-def _compress(original, dtype, MVUE24, mask, rand):
+def _panel_width(dtype):
+    """Dense columns per panel: 128 bytes of the value dtype."""
+    return 128 // torch.empty((), dtype=dtype).element_size()
+
+
+def _to_canonical(values, meta, m, n):
+    """Panel-layout storage -> canonical (values [m, n/2], meta [m, n/16 | n/32])."""
+    kp = _panel_width(values.dtype)
+    v = values.view(n // kp, m, kp // 2).permute(1, 0, 2).reshape(m, n // 2)
+    mt = meta.view(n // kp, m, 4).permute(1, 0, 2).reshape(m, -1)
+    return v, mt
+
+
+def _compress(original, dtype, MVUE24, mask, rand, panel):
     """One allocation of numel*cf/16 elements: values first, metadata in the tail
-    (reference :215-243); then the HIP prune+compress kernel."""
+    (reference :215-243); then the HIP prune+compress kernel.  Returns flat storage views."""
     m, n = original.shape
     cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[dtype]
     buf = torch.empty((original.nelement() * cfg.compression_factor // 16,), dtype=dtype, device=original.device)
-    values = buf[: m * n // 2].view(m, n // 2)
-    meta = buf[m * n // 2:].view(_indices_dtype(dtype)).view(m, -1)
+    values = buf[: m * n // 2]
+    meta = buf[m * n // 2:].view(_indices_dtype(dtype))
 
     dense = N.as_matrix(original)
     layout, ld = N.layout_of(dense)
@@ -71,16 +87,16 @@ def _compress(original, dtype, MVUE24, mask, rand):
     N.check(N.lib().tf24_prune_compress(
         dense.data_ptr(), N.dtype_code(dense.dtype), layout, ld, m, n, mode,
         N.ptr(mask_t), mask_code, mask_ld, N.ptr(rand_t), rand_ld,
-        values.data_ptr(), N.dtype_code(dtype), meta.data_ptr(), N.stream_ptr()))
+        values.data_ptr(), N.dtype_code(dtype), meta.data_ptr(),
+        N.COMPRESSED_PANEL if panel else N.COMPRESSED_CANONICAL, N.stream_ptr()))
     return values, meta
 
 
 def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, activation=N.ACT_NONE):
     """sparse_first: out = S @ dense  (S [n,k], dense [k,j])  -> [n, j]
        otherwise   : out = dense @ S^T (dense [j,k])          -> [j, n]"""
-    values, meta = sparse.sparse_tensor_cutlass, sparse.meta_tensor_cutlass
-    n, half_k = values.shape
-    k = 2 * half_k
+    values, meta = sparse._store_values, sparse._store_meta
+    n, k = sparse._store_shape
     if dense.dtype != values.dtype:
         raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
     dense = N.as_matrix(dense)
@@ -103,7 +119,7 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
         if bias.numel() != n:
             raise RuntimeError(f"bias must have {n} elements, got {bias.numel()}")
     N.check(N.lib().tf24_spmm(
-        values.data_ptr(), meta.data_ptr(), N.dtype_code(values.dtype), n, k,
+        values.data_ptr(), meta.data_ptr(), sparse._store_layout, N.dtype_code(values.dtype), n, k,
         dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.dtype_code(out_dtype), c_layout, out.stride(0),
         N.ptr(bias), float(scale), activation, N.stream_ptr()))
     return out
@@ -122,6 +138,8 @@ class SparseSemiStructuredTensor(torch.Tensor):
     _PROTOTYPE_WARNING_SHOWN = False
     # output dtype of fp8 products (the reference's CUTLASS path returns float32)
     _FP8_OUT_DTYPE = torch.float32
+    # store freshly compressed tensors in the SMFMAC panel layout (False: canonical row-major)
+    _PANEL_LAYOUT = True
 
     @staticmethod
     def __new__(cls, original_tensor: Optional[torch.Tensor], original_shape: Optional[torch.Size] = None,
@@ -173,26 +191,63 @@ class SparseSemiStructuredTensor(torch.Tensor):
                                    f"({cfg.sparse_min_rows}, {cfg.sparse_min_cols})")
             if mask is not None and MVUE24:
                 raise RuntimeError("Error using MVUE24 with mask is not supported! ")
-            compressed_tensor_cusparselt = None
-            sparse_tensor_cutlass, meta_tensor_cutlass = _compress(original_tensor, dtype, MVUE24, mask, rand)
+            panel = bool(self._PANEL_LAYOUT)
+            values, meta = _compress(original_tensor, dtype, MVUE24, mask, rand, panel)
+            self._set_storage(values, meta, (m, n), N.COMPRESSED_PANEL if panel else N.COMPRESSED_CANONICAL)
+        elif sparse_tensor_cutlass is not None:
+            # built from canonical pieces (values [m, k/2], nibble metadata)
+            mm, half = sparse_tensor_cutlass.shape
+            self._set_storage(sparse_tensor_cutlass.contiguous().view(-1), meta_tensor_cutlass.contiguous().view(-1),
+                              (mm, 2 * half), N.COMPRESSED_CANONICAL)
+        else:
+            self._set_storage(None, None, None, N.COMPRESSED_CANONICAL)
         self.original_tensor = None
-        self.compressed_tensor_cusparselt = compressed_tensor_cusparselt
-        self.sparse_tensor_cutlass = sparse_tensor_cutlass
-        self.meta_tensor_cutlass = meta_tensor_cutlass
+        self.compressed_tensor_cusparselt = None
         self.transposed = transposed
         self.original_shape = original_shape
 
+    def _set_storage(self, values, meta, shape, layout):
+        self._store_values, self._store_meta = values, meta       # flat device tensors
+        self._store_shape, self._store_layout = shape, layout     # (m, k) of the untransposed matrix
+        self._canonical = None
+
+    def _canonical_pair(self):
+        if self._canonical is None:
+            m, n = self._store_shape
+            if self._store_layout == N.COMPRESSED_PANEL:
+                self._canonical = _to_canonical(self._store_values, self._store_meta, m, n)
+            else:
+                self._canonical = (self._store_values.view(m, n // 2), self._store_meta.view(m, -1))
+        return self._canonical
+
+    @property
+    def sparse_tensor_cutlass(self):
+        """Kept values, canonical [m, k/2] (the reference's attribute name)."""
+        return None if self._store_values is None else self._canonical_pair()[0]
+
+    @property
+    def meta_tensor_cutlass(self):
+        """Canonical nibble metadata [m, k/16] int16 or [m, k/32] int32."""
+        return None if self._store_values is None else self._canonical_pair()[1]
+
     def __tensor_flatten__(self):
-        return ["sparse_tensor_cutlass", "meta_tensor_cutlass"], (self.original_shape, self.transposed)
+        return ["_store_values", "_store_meta"], (self.original_shape, self.transposed, self._store_shape, self._store_layout)
 
     @staticmethod
     def __tensor_unflatten__(inner_tensors, meta, outer_size, outer_stride):
-        original_shape, transposed = meta
+        original_shape, transposed, store_shape, store_layout = meta
         if len(inner_tensors) != 2:
             raise RuntimeError(f"Expected 2 inner tensors but got {len(inner_tensors)}")
-        return SparseSemiStructuredTensor(
-            None, original_shape=original_shape, sparse_tensor_cutlass=inner_tensors["sparse_tensor_cutlass"],
-            meta_tensor_cutlass=inner_tensors["meta_tensor_cutlass"], transposed=transposed)
+        return SparseSemiStructuredTensor._from_storage(
+            inner_tensors["_store_values"], inner_tensors["_store_meta"], store_shape, store_layout, original_shape, transposed)
+
+    @classmethod
+    def _from_storage(cls, values, meta, store_shape, store_layout, shape, transposed):
+        m, n = store_shape
+        out = cls(None, original_shape=shape, sparse_tensor_cutlass=values.view(m, n // 2), meta_tensor_cutlass=meta,
+                  transposed=transposed, dtype=values.dtype)
+        out._set_storage(values, meta, store_shape, store_layout)
+        return out
 
     def __repr__(self) -> str:  # type: ignore[override]
         return (f"SparseSemiStructuredTensor(shape={self.shape}, transposed={self.transposed}"
@@ -201,9 +256,8 @@ class SparseSemiStructuredTensor(torch.Tensor):
     __torch_function__ = torch._C._disabled_torch_function_impl
 
     def _clone_view(self, shape, transposed):
-        return SparseSemiStructuredTensor(
-            None, original_shape=shape, sparse_tensor_cutlass=self.sparse_tensor_cutlass,
-            meta_tensor_cutlass=self.meta_tensor_cutlass, transposed=transposed, dtype=self.dtype)
+        return SparseSemiStructuredTensor._from_storage(
+            self._store_values, self._store_meta, self._store_shape, self._store_layout, shape, transposed)
 
     def _pad_tensor_for_matmul(self, original_tensor: torch.Tensor) -> torch.Tensor:
         """Zero-pads a 2-d dense operand to the multiples the kernel wants (reference :351-368)."""
@@ -270,11 +324,11 @@ class SparseSemiStructuredTensor(torch.Tensor):
 
     def to_dense(self):
         """Decompress to a dense [m, k] tensor of the value dtype (reference :554-572)."""
-        values, meta = self.sparse_tensor_cutlass, self.meta_tensor_cutlass
-        m, half_k = values.shape
-        out = torch.empty((m, 2 * half_k), dtype=values.dtype, device=values.device)
-        N.check(N.lib().tf24_decompress(values.data_ptr(), N.dtype_code(values.dtype), meta.data_ptr(), m, 2 * half_k,
-                                        out.data_ptr(), N.stream_ptr()))
+        values, meta = self._store_values, self._store_meta
+        m, k = self._store_shape
+        out = torch.empty((m, k), dtype=values.dtype, device=values.device)
+        N.check(N.lib().tf24_decompress(values.data_ptr(), N.dtype_code(values.dtype), meta.data_ptr(), self._store_layout,
+                                        m, k, out.data_ptr(), N.stream_ptr()))
         return out
 
     def indices_cutlass(self):

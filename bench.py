@@ -67,11 +67,11 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
 
     def magnitude(i):
         N.check(lib.tf24_prune_compress(W[i].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MAGNITUDE, None, N.U8, 0,
-                                        None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), st))
+                                        None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
 
     def mvue(i):
         N.check(lib.tf24_prune_compress(W[i].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MVUE, None, N.U8, 0,
-                                        U[i].data_ptr(), k, values[i].data_ptr(), N.F16, meta[i].data_ptr(), st))
+                                        U[i].data_ptr(), k, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
 
     def transposable(i):
         N.check(lib.tf24_transposable_mask(W[i].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, 1, sp[i].data_ptr(),
@@ -85,7 +85,7 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
 
     def mask_compress(i):
         N.check(lib.tf24_prune_compress(P[i].data_ptr(), N.F32, N.ROW_MAJOR, k, m, k, N.PRUNE_MASK, bmask[i].data_ptr(), N.U8, k,
-                                        None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), st))
+                                        None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
 
     def copy(i):
         sp[i].copy_(W[i])

@@ -55,6 +55,18 @@ typedef enum {
 
 typedef enum { TF24_ACT_NONE = 0, TF24_ACT_RELU = 1, TF24_ACT_SILU = 2 } tf24_activation;
 
+/*
+ * Storage of a compressed [m,k] matrix (values + metadata).
+ *   CANONICAL  values [m, k/2] row-major, metadata [m, k/8 bytes] row-major (the interchange form).
+ *   PANEL      the SMFMAC-native form the matmul streams: the k axis is cut into panels of
+ *              KP = 128/sizeof(value) dense columns (64 for 16-bit values, 128 for fp8), i.e. the
+ *              64 value bytes and KP/8 metadata bytes one row contributes to one LDS stage;
+ *              values [k/KP][m][64 bytes], metadata [k/KP][m][KP/8 bytes].  A 256-row tile of one
+ *              stage is then a single contiguous 16 KB (+2/4 KB) run, copied to LDS with full-line
+ *              GLOBAL_LOAD_LDS_DWORDX4.  Inside a row of a panel the bytes are the canonical ones.
+ */
+typedef enum { TF24_COMPRESSED_CANONICAL = 0, TF24_COMPRESSED_PANEL = 1 } tf24_compressed_layout;
+
 /* Library version string, e.g. "tf24 0.1.0 gfx950". Host only. */
 const char* tf24_version(void);
 
@@ -71,15 +83,15 @@ const char* tf24_last_error(void);
  *   mask       [m,k] mask_dtype (U8|F16|BF16|F32), nonzero = kept, same layout, leading dim mask_ld
  *   rand       [m,k] F32 uniforms in [0,1), same layout, leading dim rand_ld; group g of row r
  *              uses rand[r,4g] and rand[r,4g+1]
- *   values     [m,k/2] out_dtype (F16|BF16|E4M3), row-major contiguous
- *   meta       canonical int16 [m,k/16] (F16|BF16) or int32 [m,k/32] (E4M3), row-major contiguous
+ *   values     m*k/2 elements of out_dtype (F16|BF16|E4M3) in out_layout
+ *   meta       m*k/8 bytes in out_layout (canonical: int16 [m,k/16] for 16-bit values, int32 [m,k/32] for E4M3)
  * Shape rules (sparse/semi_structured.py:24-30,188-200): m % 32 == 0, k % 64 == 0 for 16-bit
  * values, k % 128 == 0 for 8-bit values.
  */
 int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
                         int mode, const void* mask, int mask_dtype, int64_t mask_ld,
                         const float* rand, int64_t rand_ld,
-                        void* values, int out_dtype, void* meta, void* stream);
+                        void* values, int out_dtype, void* meta, int out_layout, void* stream);
 
 /* The argument checks of tf24_prune_compress without touching the GPU (pointers are only
  * tested for NULL-ness through the has_* flags). Host only. */
@@ -90,10 +102,10 @@ int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld, int64_t m
 /*
  * Compressed -> dense.  Replaces _sparse_semi_structured_to_dense_kernel
  * (sparse/_semi_structured_conversions.py:1163-1274) used by SparseSemiStructuredTensor.to_dense
- * (sparse/semi_structured.py:554-572).  values [m,k/2] dtype, meta canonical, dense_out [m,k]
- * row-major contiguous of the same dtype.
+ * (sparse/semi_structured.py:554-572).  values / meta in `layout`, dense_out [m,k] row-major
+ * contiguous of the same dtype.
  */
-int tf24_decompress(const void* values, int dtype, const void* meta, int64_t m, int64_t k,
+int tf24_decompress(const void* values, int dtype, const void* meta, int layout, int64_t m, int64_t k,
                     void* dense_out, void* stream);
 
 /*
@@ -138,7 +150,7 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * Replaces sparse.cutlass.my_sparse_semi_structured_linear
  * (sparse/csrc/mySparseSemiStructuredLinear_cuda.cu:498-817, CUTLASS SparseGemm :61-76),
  * bound at sparse/sparse_semi_structured_linear.py:4-5.
- *   a_values [n_sparse,k/2], a_meta canonical; dtype F16|BF16|E4M3 (B has the same dtype)
+ *   a_values, a_meta  the compressed operand in a_layout; dtype F16|BF16|E4M3 (B has the same dtype)
  *   b          dense operand, n_dense "columns" j: b_layout TF24_ROW_MAJOR means B is stored
  *              [n_dense, k] (k contiguous, element (k,j) at j*ldb + k: the X of X.W^T);
  *              TF24_COL_MAJOR means stored [k, n_dense] (element (k,j) at k*ldb + j)
@@ -149,7 +161,7 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * Shape rules (.cu:101-109): n_sparse % 32 == 0, k % 64 == 0 (16-bit) / 128 (8-bit),
  * n_dense % 8 == 0 (16-bit) / 16 (8-bit).
  */
-int tf24_spmm(const void* a_values, const void* a_meta, int dtype, int64_t n_sparse, int64_t k,
+int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,
               const void* b, int b_layout, int64_t ldb, int64_t n_dense,
               void* c, int out_dtype, int c_layout, int64_t ldc,
               const void* bias, float scale, int activation, void* stream);

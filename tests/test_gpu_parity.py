@@ -57,6 +57,36 @@ def test_magnitude_compress(cuda, shape, in_dtype, out_dtype, col_major):
     assert_same(s.to_dense(), oracle.decompress24(want_v, want_m), "to_dense")
 
 
+@pytest.mark.parametrize("out_dtype", [F16, E4M3])
+@pytest.mark.parametrize("col_major", [False, True])
+def test_canonical_and_panel_storage_agree(cuda, out_dtype, col_major):
+    """The same tensor compressed into the canonical and into the panel layout: identical
+    values()/indices()/to_dense() and identical products."""
+    import sparse
+    cls = sparse.SparseSemiStructuredTensor
+    w = randn((96, 384), F16, 18)
+    x = randn((40 if out_dtype == F16 else 48, 384), F16, 19).to(cuda)
+    want_v, want_m = oracle.compress24(w, out_dtype=out_dtype)
+    outs = []
+    try:
+        for panel in (True, False):
+            cls._PANEL_LAYOUT = panel
+            s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major), dtype=out_dtype)
+            assert s._store_layout == (1 if panel else 0)
+            assert_same(s.values(), want_v, f"values panel={panel}")
+            assert_same(s.indices(), want_m, f"meta panel={panel}")
+            assert_same(s.to_dense(), oracle.decompress24(want_v, want_m), f"to_dense panel={panel}")
+            outs.append(torch.mm(x.to(out_dtype), s.t()))
+            outs.append(torch.mm(s, x.to(out_dtype).t().contiguous()))
+    finally:
+        cls._PANEL_LAYOUT = True
+    assert_same(outs[0], outs[2], "x.W^T panel vs canonical")
+    assert_same(outs[1], outs[3], "W.x^T panel vs canonical")
+    # round trip through the canonical constructor arguments
+    s2 = cls(None, original_shape=s.shape, sparse_tensor_cutlass=s.values(), meta_tensor_cutlass=s.indices(), dtype=out_dtype)
+    assert_same(torch.mm(x.to(out_dtype), s2.t()), outs[0], "rebuilt from canonical pieces")
+
+
 def test_docstring_known_answer(cuda):
     import sparse
     a = torch.tensor([0.0, 0.0, 1.0, 1.0]).tile((128, 32)).half().to(cuda)
@@ -316,7 +346,7 @@ def test_dispatch_rules(cuda):
     w = _small_ints((32, 64), 58).half().to(cuda)
     s = sparse.to_sparse_semi_structured(w)
     assert s.t().transposed and s.t().shape == (64, 32) and not s.t().t().transposed
-    assert s.detach().values().data_ptr() == s.values().data_ptr()
+    assert s.detach()._store_values.data_ptr() == s._store_values.data_ptr()
     x = torch.ones(8, 64, dtype=F16, device=cuda)
     with pytest.raises(NotImplementedError):
         torch.mm(x, s)                                     # second operand must be transposed
