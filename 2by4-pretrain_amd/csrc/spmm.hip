@@ -148,9 +148,21 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 
 
 // ------------------------------------------------------------------------------------------
-// Tiled kernel (B with k contiguous): 512 lanes = 8 waves (2 along i x 4 along j) compute a
-// 256(i) x 256(j) tile; a wave owns 128 x 64 = 4 x 2 instructions of 32x32.  Operands are staged
-// through LDS in stages of 128 bytes of dense k per row (two instruction steps).
+// Tiled kernel: A in the panel layout, B with k contiguous.
+//
+// A block computes a 256(i) x 256(j) tile with V_SMFMAC_F32_32X32X32_{F16,BF16} / 32X32X64_FP8.
+// Two wave arrangements (template parameter Cfg):
+//   Cfg8: 8 waves (2 along i x 4 along j), wave tile 128 x 64 = 4 x 2 instructions, 2 waves per SIMD
+//   Cfg4: 4 waves (2 x 2), wave tile 128 x 128 = 4 x 4 instructions, 256 accumulator registers,
+//         1 wave per SIMD: fewer LDS reads per instruction, but measured slower (kept for reference)
+// Operands go global -> LDS directly (GLOBAL_LOAD_LDS_DWORDX4: lane l of a wave writes
+// LDS[base + 16*l], a wave fills 1 KB of contiguous LDS) through a ring of three stage buffers of
+// 128 bytes of dense k per row (two instruction steps): while stage s is multiplied, the copies of
+// stages s+1 and s+2 are in flight.  LDS rows are unpadded; bank conflicts are avoided by
+// XOR-swizzling the 16-byte chunk index with row bits (B: chunk ^ ((row>>1)&7) in 128-byte rows,
+// A: chunk ^ ((row>>2)&3) in 64-byte rows), applied on the global side of the copy and again in the
+// fragment reads.  The three buffers are separate LDS objects and the stage loop is unrolled by
+// three, so that every LDS access names its buffer statically.
 // Workgroup ids are remapped so that the 8 XCDs (ids are dealt round-robin) each walk a
 // contiguous range of tiles in an 8-tile-high grouped raster: the ~32 tiles resident on an XCD
 // form an 8 x 4 patch that shares A rows and B columns in that XCD's L2.
@@ -172,29 +184,27 @@ template <> struct mma32<e4m3_t> {
   }
 };
 
-struct TileCfg {
-  static constexpr int THREADS = 512;
-  static constexpr int BI = 256, BJ = 256;       // block tile
-  static constexpr int WI = 128, WJ = 64;        // wave tile
-  static constexpr int TI = WI / 32, TJ = WJ / 32;
+template <int WAVES_J_, int TJ_>
+struct TileCfgT {
+  static constexpr int WAVES_I = 2, WAVES_J = WAVES_J_;
+  static constexpr int NW = WAVES_I * WAVES_J;
+  static constexpr int THREADS = 64 * NW;
+  static constexpr int TI = 4, TJ = TJ_;         // 32x32 instructions per wave
+  static constexpr int WI = 32 * TI, WJ = 32 * TJ;
+  static constexpr int BI = WI * WAVES_I, BJ = WJ * WAVES_J;
+  static_assert(BI == 256 && BJ == 256, "stage buffers are sized for 256 x 256 tiles");
   static constexpr int KB = 128;                 // bytes of dense k per row per stage
   static constexpr int STEPS = KB / 64;          // instruction steps per stage
   static constexpr int A_ROW = KB / 2;           // LDS bytes per row per stage: compressed values
   static constexpr int B_ROW = KB;               //                              dense operand
   static constexpr int GH = 8;                   // raster group height in tiles along i
+  static constexpr int NB = BJ * B_ROW / 1024 / NW;   // 1 KB copies per wave per stage: B
+  static constexpr int NA = BI * A_ROW / 1024 / NW;   //                                 A values
 };
+using Cfg8 = TileCfgT<4, 2>;
+using Cfg4 = TileCfgT<2, 4>;
+using TiledCfg = Cfg8;
 
-// ------------------------------------------------------------------------------------------
-// Pipelined kernel: same tiling as spmm_tiled, but operands go global -> LDS directly
-// (GLOBAL_LOAD_LDS_DWORDX4: lane l of a wave writes LDS[base + 16*l], so a wave fills 1 KB of
-// contiguous LDS) through a ring of three stage buffers: while stage s is multiplied, the loads
-// of stages s+1 and s+2 are in flight, which covers the L2/HBM latency that one stage of math
-// cannot.  LDS rows are unpadded; bank conflicts are avoided by XOR-swizzling the 16-byte chunk
-// index with row bits (B: chunk ^ ((row>>1)&7) in 128-byte rows, A: chunk ^ ((row>>2)&3) in
-// 64-byte rows), applied on the global side of the copy and again in the fragment reads.
-// The three buffers are separate LDS objects and the stage loop is unrolled by three, so that
-// every LDS access names its buffer statically.
-// ------------------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // The copies are issued from inline assembly so that the compiler's wait-count insertion does not
@@ -207,20 +217,24 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p) {
 __device__ __forceinline__ void g2l16(const uint8_t* g, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
 }
-__device__ __forceinline__ void g2l4(const uint8_t* g, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
+// s_waitcnt vmcnt(N) + s_barrier with a compile-time N (a bare s_barrier: __syncthreads() would add
+// a fence that drains every outstanding copy)
+template <int N>
+__device__ __forceinline__ void wait_copies_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <typename T, typename OutT, bool C_JMAJOR, bool PANEL>
-__global__ void __launch_bounds__(TileCfg::THREADS)
+template <typename T, typename OutT, bool C_JMAJOR, typename C>
+__global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
           OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act,
           int tiles_i, int tiles_j) {
-  using C = TileCfg;
   constexpr int ES = sizeof(T);
   constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
   constexpr int M_STEP = M_ROW / C::STEPS;
+  constexpr int M_COPIES = C::BI * M_ROW / 1024;            // 1 KB copies per stage: metadata (2 or 4)
+  static_assert(M_COPIES <= C::NW, "one metadata copy per wave at most");
   constexpr int A_STAGE = C::BI * C::A_ROW, B_STAGE = C::BJ * C::B_ROW, M_STAGE = C::BI * M_ROW;
   __shared__ __attribute__((aligned(1024))) uint8_t s_a0[A_STAGE];
   __shared__ __attribute__((aligned(1024))) uint8_t s_a1[A_STAGE];
@@ -232,6 +246,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   __shared__ __attribute__((aligned(1024))) uint8_t s_m1[M_STAGE];
   __shared__ __attribute__((aligned(1024))) uint8_t s_m2[M_STAGE];
 
+  // ---- XCD-aware tile assignment
   const int ntiles = tiles_i * tiles_j;
   const int per_xcd = (ntiles + 7) / 8;
   const int bid = blockIdx.x;
@@ -247,74 +262,47 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wi = wave >> 2, wj = wave & 3;
+  const int wi = wave / C::WAVES_J, wj = wave % C::WAVES_J;
   const int l32 = lane & 31, lh = lane >> 5;
-
-  const int64_t a_pitch = (k / 2) * ES;
-  const int64_t m_pitch = k / 8;
   const int nstages = (int)((k * ES) / C::KB);
 
-  // ---- per-lane global sources of the copies (stage 0), LDS destinations are wave-uniform
-  const uint8_t* gb[4];
-  const uint8_t* ga[2];
-  const uint8_t* gm;
+  // ---- per-lane global sources of the copies (stage 0); LDS destinations are wave-uniform.
+  // B: copy q of a wave brings 8 rows x 128 bytes; lane -> (row, swizzled chunk).
+  // A: stage st of rows i0..i0+255 is one contiguous run of 256*64 value bytes at (st*n_sparse + i0)*64
+  //    (and 256*M_ROW metadata bytes): copy q brings 16 rows x 64 bytes.
+  const uint8_t* gb[C::NB];
+  const uint8_t* ga[C::NA];
 #pragma unroll
-  for (int q = 0; q < 4; q++) {
-    const int row = (wave * 4 + q) * 8 + (lane >> 3);
+  for (int q = 0; q < C::NB; q++) {
+    const int row = (wave * C::NB + q) * 8 + (lane >> 3);
     const int ch = (lane & 7) ^ ((row >> 1) & 7);
     gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16;
   }
-  // A and its metadata.  Canonical layout: rows strided by the row pitch, 64 value bytes (4 chunks)
-  // and M_ROW metadata bytes per row per stage.  Panel layout: stage st of rows i0..i0+255 is one
-  // contiguous run of 256*64 value bytes at (st*n_sparse + i0)*64 and 256*M_ROW metadata bytes.
-  int64_t a_stage_stride, m_stage_stride;
-  bool has_meta_copy = true;
-  if constexpr (PANEL) {
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
-      const int row = (wave * 2 + q) * 16 + (lane >> 2);
-      const int ch = (lane & 3) ^ ((row >> 2) & 3);
-      ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16;
-    }
-    // metadata: 1 KB per copy = 128 rows (M_ROW 8) or 64 rows (M_ROW 16): waves 0..(2 or 4)-1
-    constexpr int M_COPIES = C::BI * M_ROW / 1024;
-    has_meta_copy = wave < M_COPIES;
+  for (int q = 0; q < C::NA; q++) {
+    const int row = (wave * C::NA + q) * 16 + (lane >> 2);
+    const int ch = (lane & 3) ^ ((row >> 2) & 3);
+    ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16;
+  }
+  const bool has_meta_copy = wave < M_COPIES;
+  const uint8_t* gm;
+  {
     const int row = (wave % M_COPIES) * (1024 / M_ROW) + lane * 16 / M_ROW;
     // a 16-byte copy spans 16/M_ROW rows: clamp so that it never reaches past the last row
     gm = a_meta + min(i0 + row, n_sparse - 16 / M_ROW) * M_ROW + (lane * 16) % M_ROW;
-    a_stage_stride = n_sparse * 64;
-    m_stage_stride = n_sparse * M_ROW;
-  } else {
-#pragma unroll
-    for (int q = 0; q < 2; q++) {
-      const int row = (wave * 2 + q) * 16 + (lane >> 2);
-      const int ch = (lane & 3) ^ ((row >> 2) & 3);
-      ga[q] = a_values + min(i0 + row, n_sparse - 1) * a_pitch + ch * 16;
-    }
-    if constexpr (M_ROW == 8) {
-      const int row = wave * 32 + (lane >> 1);
-      gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch + (lane & 1) * 4;
-    } else {
-      const int row = (wave & 3) * 64 + lane;
-      gm = a_meta + min(i0 + row, n_sparse - 1) * m_pitch;
-    }
-    a_stage_stride = C::A_ROW;
-    m_stage_stride = M_ROW;
   }
-  // copy number q (0..6) of a stage: 4 x B, 2 x A, 1 x metadata
+  const int64_t a_stage_stride = n_sparse * 64, m_stage_stride = n_sparse * M_ROW;
+  constexpr int NCOPY = C::NB + C::NA + 1;       // copies per wave per stage (one less without metadata copy)
+
   auto issue_one = [&](int q, int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
-    if (q < 4) g2l16(gb[q] + (int64_t)st * C::B_ROW, lds_offset(sb) + (wave * 4 + q) * 1024);
-    else if (q < 6) g2l16(ga[q - 4] + (int64_t)st * a_stage_stride, lds_offset(sa) + (wave * 2 + q - 4) * 1024);
-    else if constexpr (PANEL) {
-      if (has_meta_copy) g2l16(gm + (int64_t)st * m_stage_stride, lds_offset(sm) + wave * 1024);
-    } else if constexpr (M_ROW == 8) g2l4(gm + (int64_t)st * M_ROW, lds_offset(sm) + wave * 256);
-    else g2l16(gm + (int64_t)st * M_ROW, lds_offset(sm) + (wave & 3) * 1024);    // waves 4-7 repeat the copy of waves 0-3
+    if (q < C::NB) g2l16(gb[q] + (int64_t)st * C::B_ROW, lds_offset(sb) + (wave * C::NB + q) * 1024);
+    else if (q < C::NB + C::NA) g2l16(ga[q - C::NB] + (int64_t)st * a_stage_stride, lds_offset(sa) + (wave * C::NA + q - C::NB) * 1024);
+    else if (has_meta_copy) g2l16(gm + (int64_t)st * m_stage_stride, lds_offset(sm) + wave * 1024);
   };
   auto issue = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
 #pragma unroll
-    for (int q = 0; q < 7; q++) issue_one(q, st, sa, sb, sm);
+    for (int q = 0; q < NCOPY; q++) issue_one(q, st, sa, sb, sm);
   };
-  constexpr int LOADS_PER_STAGE = 7;   // copies per wave per stage (6 for panel-layout waves without a metadata copy)
 
   float16v acc[C::TI][C::TJ];
 #pragma unroll
@@ -336,10 +324,13 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   }
   const int m_off = a_row * M_ROW + lh * (M_STEP / 2);
 
-  // Math of one stage.  The copies of the stage two ahead (into the buffer freed by the barrier) are
-  // issued one at a time between the matrix instructions: issued in a burst right after the barrier
-  // they would queue up in the texture-address unit and hold back every wave's fragment reads.
-  auto compute = [&](const uint8_t* sa, const uint8_t* sb, const uint8_t* sm, bool prefetch, int pst, uint8_t* na, uint8_t* nb,
+  // ---- one stage: barrier (the stage's copies have landed and every wave is done with the buffer
+  // that is refilled next), then the two instruction steps.  The copies of stage+2 are spread
+  // between the matrix instructions: issued in a burst they would queue in the texture-address unit
+  // and hold back the fragment reads behind them.  (Double-buffering the fragments in registers
+  // across the barrier, and 128x128 wave tiles with one wave per SIMD, were both measured slower:
+  // the two waves of a SIMD already hide each other's LDS latency.)
+  auto compute = [&](const uint8_t* sa, const uint8_t* sb, const uint8_t* sm, bool copies, int pst, uint8_t* na, uint8_t* nb,
                      uint8_t* nm) {
 #pragma unroll
     for (int step = 0; step < C::STEPS; step++) {
@@ -362,23 +353,26 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
       for (int ti = 0; ti < C::TI; ti++) {
 #pragma unroll
         for (int tj = 0; tj < C::TJ; tj++) acc[ti][tj] = mma32<T>::run(af[ti], bf[tj], acc[ti][tj], idx[ti]);
-        const int q = step * C::TI + ti;           // 8 slots per stage, 7 copies
-        if (q < 7 && prefetch) {
-          __builtin_amdgcn_sched_barrier(0);
-          issue_one(q, pst, na, nb, nm);
-          __builtin_amdgcn_sched_barrier(0);
+        // one or two copies after each row of instructions
+        constexpr int PER_SLOT = (NCOPY + C::STEPS * C::TI - 1) / (C::STEPS * C::TI);
+#pragma unroll
+        for (int u = 0; u < PER_SLOT; u++) {
+          const int q = (step * C::TI + ti) * PER_SLOT + u;
+          if (q < NCOPY && copies) {
+            __builtin_amdgcn_sched_barrier(0);
+            issue_one(q, pst, na, nb, nm);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
     }
   };
-
-  // one pipeline step: stage `st` lives in (sa,sb,sm); the buffer freed by stage st-1 is (na,nb,nm)
+  // stage `st` lives in (sa,sb,sm); the buffer freed by stage st-1 is (na,nb,nm) and receives stage st+2
   auto pipe_step = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm, uint8_t* na, uint8_t* nb, uint8_t* nm) {
-    // loads of stage st were issued two steps ago; at most the loads of stage st+1 may still fly
-    // (a bare s_barrier: __syncthreads() would add a fence that drains every outstanding copy)
-    if (st + 1 >= nstages) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else if (has_meta_copy) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LOADS_PER_STAGE - 1) : "memory");
+    // the copies of stage st were issued two stages ago; only those of stage st+1 may still fly
+    if (st + 1 >= nstages) wait_copies_and_barrier<0>();
+    else if (has_meta_copy) wait_copies_and_barrier<NCOPY>();
+    else wait_copies_and_barrier<NCOPY - 1>();
     compute(sa, sb, sm, st + 2 < nstages, st + 2, na, nb, nm);
   };
 
@@ -393,48 +387,88 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   if (st < nstages) { pipe_step(st, s_a0, s_b0, s_m0, s_a2, s_b2, s_m2); st++; }
   if (st < nstages) { pipe_step(st, s_a1, s_b1, s_m1, s_a0, s_b0, s_m0); st++; }
 
+  // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
+  // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
+  // (8 bytes) in 32 different output rows, so direct stores would touch 32 lines per instruction.
+  // Instead every wave stages 64(j) x 128(i) pieces of its sub-tile in a private 16 KB slice of the
+  // now idle B stage buffers (256-byte rows, 16-byte chunks XOR-swizzled with the row) and streams
+  // them out as four full 256-byte row segments per instruction.
+  if constexpr (C_JMAJOR && sizeof(OutT) == 2) {
+    __syncthreads();                                          // every wave is done with the stage buffers
+    uint8_t* stage = wave < 2 ? s_b0 + wave * 16384 : wave < 4 ? s_b1 + (wave - 2) * 16384
+                   : wave < 6 ? s_b2 + (wave - 4) * 16384 : wave == 6 ? s_a0 : s_a1;
+    const int rr = lane >> 4, chr = lane & 15;
+    const int64_t icol = i0 + wi * C::WI + chr * 8;
 #pragma unroll
-  for (int ti = 0; ti < C::TI; ti++)
+    for (int half = 0; half < C::TJ / 2; half++) {            // 64 output rows (j) per pass
 #pragma unroll
-    for (int tj = 0; tj < C::TJ; tj++) {
-      const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
+      for (int ti = 0; ti < C::TI; ti++)
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
-        if (col >= n_dense || row >= n_sparse) continue;
-        OutT o[4];
+        for (int t2 = 0; t2 < 2; t2++) {
+          const int tj = half * 2 + t2;
+          const int jl = t2 * 32 + l32;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          float v = acc[ti][tj][g * 4 + r] * scale;
-          if (bias) v += to_float(bias[row + r]);
-          o[r] = from_float<OutT>(apply_act(v, act));
+          for (int g = 0; g < 4; g++) {
+            const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+            OutT o[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              float v = acc[ti][tj][g * 4 + r] * scale;
+              if (bias && row < n_sparse) v += to_float(bias[row + r]);
+              o[r] = from_float<OutT>(apply_act(v, act));
+            }
+            const int ch = ti * 4 + g;
+            *reinterpret_cast<Pack<OutT, 4>*>(stage + jl * 256 + ((ch ^ (jl & 15)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+          }
         }
-        if constexpr (C_JMAJOR) {
-          *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
-        } else {
 #pragma unroll
-          for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
-        }
+      for (int it = 0; it < 16; it++) {
+        const int jl = it * 4 + rr;
+        const int64_t jrow = j0 + wj * C::WJ + half * 64 + jl;
+        const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 256 + ((chr ^ (jl & 15)) * 16));
+        if (jrow < n_dense && icol < n_sparse) *reinterpret_cast<int4v*>(c + jrow * ldc + icol) = v;
       }
     }
+  } else {
+#pragma unroll
+    for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+      for (int tj = 0; tj < C::TJ; tj++) {
+        const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+          if (col >= n_dense || row >= n_sparse) continue;
+          OutT o[4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            float v = acc[ti][tj][g * 4 + r] * scale;
+            if (bias) v += to_float(bias[row + r]);
+            o[r] = from_float<OutT>(apply_act(v, act));
+          }
+          if constexpr (C_JMAJOR) {
+            *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
+          }
+        }
+      }
+  }
 }
 
-template <typename T, typename OutT>
-int launch_tiled(const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
+template <typename T, typename OutT, typename C>
+int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
-  using C = TileCfg;
   const int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI), tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
   const int per_xcd = (tiles_i * tiles_j + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
-  const bool jm = c_layout == TF24_COL_MAJOR;
-#define TF24_GO(JM, PN)                                                                                                       \
-  hipLaunchKernelGGL((spmm_pipe<T, OutT, JM, PN>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, \
-                     (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j)
-  if (jm && panel) TF24_GO(true, true);
-  else if (jm) TF24_GO(true, false);
-  else if (panel) TF24_GO(false, true);
-  else TF24_GO(false, false);
-#undef TF24_GO
+  if (c_layout == TF24_COL_MAJOR)
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, true, C>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
+                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
+  else
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, false, C>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
+                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
   return check_launch("tf24_spmm");
 }
 
@@ -458,11 +492,11 @@ template <typename T>
 int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout,
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  hipStream_t s) {
-  if (b_layout == TF24_ROW_MAJOR && n_sparse >= 64 && n_dense >= 64) {
+  if (panel && b_layout == TF24_ROW_MAJOR && n_sparse >= 64 && n_dense >= 64) {
     switch (out_dtype) {
-      case TF24_F16: return launch_tiled<T, f16_t>(av, am, panel, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-      case TF24_BF16: return launch_tiled<T, bf16_t>(av, am, panel, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-      case TF24_F32: return launch_tiled<T, float>(av, am, panel, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_BF16: return launch_tiled<T, bf16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_F32: return launch_tiled<T, float, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
     }
   }
   switch (out_dtype) {
