@@ -10,6 +10,7 @@ from .decay import masked_add_
 from .dense_ops import (soft_threshold24, sparse24, MVUE24_approx,
                         soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton)
 from .sparse_linear_transpose import SparseLinearTranspose, sparse_linear_transpose
+from .sparse_semi_structured_linear import sparse_semi_structured_linear
 
 __all__ = [
     "SparseSemiStructuredTensor", "to_sparse_semi_structured",
@@ -18,4 +19,5 @@ __all__ = [
     "soft_threshold24", "sparse24", "MVUE24_approx",
     "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
     "SparseLinearTranspose", "sparse_linear_transpose",
+    "sparse_semi_structured_linear",
 ]

@@ -1,0 +1,164 @@
+"""GPU integration: SparseLinearTranspose forward/backward against a dense masked autograd model,
+a short masked-decay training loop (BASELINE config 4, reduced), and the fp8 path of config 5."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    return ((a.float() - b.float()).norm() / b.float().norm()).item()
+
+
+def test_sparse_linear_transpose_matches_dense_masked(cuda):
+    import sparse
+    torch.manual_seed(0)
+    layer = sparse.SparseLinearTranspose(256, 512, bias=True).to(cuda)
+    x = torch.randn(4, 64, 256, device=cuda, requires_grad=True)
+    y = layer(x)
+    assert y.shape == (4, 64, 512) and y.dtype == torch.float16
+    w = layer.weight.detach()
+    # the mask is the transposable one of the master weight (bit-exact with the oracle)
+    _, want_mask = oracle.transposable_mask(w.float().cpu())
+    assert layer.weight.mask.cpu().equal(want_mask)
+    wm = (w * layer.weight.mask).half()
+    y_ref = F.linear(x.detach().half(), wm, layer.bias.detach().half())
+    assert _rel(y, y_ref) < 1e-2
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    dx_ref = gy.reshape(-1, 512).float() @ wm.float()
+    assert _rel(x.grad.reshape(-1, 256), dx_ref) < 1e-2
+    db_ref = gy.reshape(-1, 512).float().sum(0)
+    assert _rel(layer.bias.grad, db_ref) < 1e-2
+    # dW is an MVUE estimate of dY^T x (pruned along the token axis): unbiased, so the mean of
+    # several draws converges to the dense gradient
+    dw_ref = gy.reshape(-1, 512).float().t() @ x.detach().reshape(-1, 256).half().float()
+    assert layer.weight.grad.shape == (512, 256)
+    single = _rel(layer.weight.grad, dw_ref)
+    draws = []
+    for _ in range(24):
+        layer.weight.grad = None
+        layer.weight.cnt = 0
+        x2 = x.detach().clone().requires_grad_(True)
+        layer(x2).backward(gy)
+        draws.append(layer.weight.grad.float())
+    mean_err = _rel(torch.stack(draws).mean(0), dw_ref)
+    assert single < 1.0 and mean_err < 0.25 and mean_err < 0.6 * single, (single, mean_err)
+
+
+def test_layer_state_machine(cuda):
+    import sparse
+    torch.manual_seed(1)
+    layer = sparse.SparseLinearTranspose(128, 128, bias=False).to(cuda)
+    w = layer.weight
+    assert (w.freq, w.cnt, w.counter, w.step, w.mode) == (40, 0, 0, 0, 'sparse')
+    x = torch.randn(32, 128, device=cuda)
+    layer(x)
+    first = w.weight_sparse
+    assert (w.cnt, w.counter, w.step) == (1, 1, 1)
+    layer(x)                                     # gradient accumulation: no recompression
+    assert w.weight_sparse is first and (w.cnt, w.counter, w.step) == (2, 1, 2)
+    w.cnt = 0                                    # what the optimizer hook does
+    layer(x)
+    assert w.weight_sparse is not first and w.counter == 2
+    w.mode = 'dense'
+    y = layer(x)
+    assert torch.allclose(y, F.linear(x, w), atol=1e-5)
+    layer.eval()
+    w.mode = 'sparse'
+    before = (w.cnt, w.counter, w.step)
+    layer(x)
+    assert (w.cnt, w.counter, w.step) == before
+
+
+def test_masked_decay_training_loop(cuda):
+    """BASELINE config 4 at reduced size: GELU MLP of two SparseLinearTranspose layers, fused
+    AdamW, masked decay alpha = 2e-4 before every optimizer step, mask refresh every 5 steps."""
+    import sparse
+    torch.manual_seed(2)
+    tokens, d, h = 512, 128, 256
+    fc, proj = sparse.SparseLinearTranspose(d, h).to(cuda), sparse.SparseLinearTranspose(h, d).to(cuda)
+    for layer in (fc, proj):
+        torch.nn.init.normal_(layer.weight, std=0.02)
+        layer.weight.freq = 5
+    params = list(fc.parameters()) + list(proj.parameters())
+    opt = torch.optim.AdamW(params, lr=3e-3, weight_decay=0.0, fused=True)
+    x = torch.randn(tokens, d, device=cuda)
+    target = torch.tanh(x @ torch.randn(d, d, device=cuda) * 0.3)
+    losses, masks = [], []
+    for step in range(20):
+        out = proj(F.gelu(fc(x)))
+        loss = F.mse_loss(out.float(), target)
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        with torch.no_grad():
+            for p in params:
+                if hasattr(p, 'mask') and p.mode == 'sparse':
+                    p.grad = p.grad.float()
+                    before = p.grad.clone()
+                    sparse.masked_add_(p.grad.data, p.data, p.mask, alpha=2e-4)
+                    want = oracle.masked_add(before.cpu(), p.data.cpu(), p.mask.cpu(), alpha=2e-4)
+                    assert p.grad.cpu().equal(want)
+                    p.cnt = 0
+        opt.step()
+        losses.append(loss.item())
+        masks.append(fc.weight.mask.clone())
+        if step % 5 == 0:       # refreshed on this forward pass from the weights before the update
+            blk = fc.weight.mask.reshape(h // 4, 4, d // 4, 4)
+            assert blk.sum(1).eq(2).all() and blk.sum(3).eq(2).all()
+    assert losses[-1] < 0.7 * losses[0], losses
+    assert masks[1].equal(masks[4]) and fc.weight.counter == 20       # constant between refreshes
+    assert all(torch.isfinite(torch.tensor(losses)))
+
+
+def test_fp8_mvue_spmm_config5_reduced(cuda):
+    """Config 5 at reduced size: per-tensor amax scaling to e4m3, B pruned by MVUE24 with seeded
+    uniforms, fp8 SMFMAC product with bf16 output, against the dense fp32 masked product."""
+    import sparse
+    g = torch.Generator().manual_seed(5)
+    A = torch.randn(512, 1024, generator=g)
+    B = torch.randn(256, 1024, generator=g)
+    U = torch.rand(256, 1024, generator=g)
+    sa, sb = 448.0 / A.abs().max(), 224.0 / B.abs().max()        # headroom: MVUE rescales kept values by up to 2x+
+    Aq = (A * sa).to(torch.float8_e4m3fn)
+    Bs = (B * sb).bfloat16()
+    want_v, want_m, mask = oracle.mvue24(Bs, U, out_dtype=torch.float8_e4m3fn)
+    s = sparse.to_sparse_semi_structured(Bs.to(cuda), MVUE24=True, rand=U.to(cuda), dtype=torch.float8_e4m3fn)
+    assert s.values().cpu().view(torch.uint8).equal(want_v.view(torch.uint8))
+    assert s.indices().cpu().equal(want_m)
+    dense_b = oracle.decompress24(want_v, want_m).float()
+    ref = (Aq.float() @ dense_b.t()) / (sa * sb)
+    out = sparse.sparse_semi_structured_linear(Aq.to(cuda), s, out_dtype=torch.bfloat16, scale=float(1.0 / (sa * sb)))
+    assert out.dtype == torch.bfloat16 and out.shape == (512, 256)
+    assert _rel(out.cpu(), ref) < 5e-2
+    # default dispatch returns float32 like the reference's CUTLASS path
+    out32 = torch.mm(Aq.to(cuda), s.t())
+    assert out32.dtype == torch.float32 and _rel(out32.cpu() / (sa * sb), ref) < 5e-2
+    # soft threshold on the bf16 operand, as config 5 applies every iteration
+    sp, mk = sparse.soft_threshold24_triton(Bs.to(cuda))
+    wsp, wmk = oracle.soft_threshold24(Bs)
+    assert sp.cpu().view(torch.int16).equal(wsp.view(torch.int16)) and mk.cpu().view(torch.int16).equal(wmk.view(torch.int16))
+
+
+def test_functional_linear_entry_point(cuda):
+    import sparse
+    g = torch.Generator().manual_seed(6)
+    w = torch.randint(-3, 4, (64, 128), generator=g).half()
+    x = torch.randint(-3, 4, (2, 9, 128), generator=g).half()
+    bias = torch.randint(-3, 4, (64,), generator=g).half()
+    mask = oracle.prune24_mask(w)
+    wm = torch.where(mask, w, torch.zeros_like(w))
+    s = sparse.to_sparse_semi_structured(w.to(cuda))
+    ref = oracle.linear_ref(x, wm, bias)
+    out = sparse.sparse_semi_structured_linear(x.to(cuda), s, bias=bias.to(cuda))
+    assert out.float().cpu().equal(ref)
+    out = sparse.sparse_semi_structured_linear(x.to(cuda), s.values(), s.indices(), bias=bias.to(cuda), activation="relu")
+    assert out.float().cpu().equal(ref.clamp_min(0))
+    out = sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="silu")
+    ref_silu = F.silu(oracle.linear_ref(x, wm))
+    assert torch.allclose(out.float().cpu(), ref_silu, rtol=2e-3, atol=2e-3)
+    with pytest.raises(RuntimeError):
+        sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="gelu")
