@@ -24,6 +24,9 @@ import torch  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_DENSE_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA; SMFMAC executes MACs at this rate
+# HBM bytes per spmm launch (mean of forward and transposed) from two rocprofv3 --pmc runs of this file:
+# FETCH_SIZE 416448 KiB + WRITE_SIZE 120832 KiB, both counters reading factor 1.00 on a copy kernel of known size
+SPMM_TRAFFIC_BYTES = (416448 + 120832) * 1024
 
 
 def _events(n):
@@ -173,29 +176,33 @@ def spmm_workload(steps, warmup):
 
 
 def cpu_baseline_spmm(threads):
-    """The oracle (pure-PyTorch port of the reference semantics) on the host cores, on a bounded
-    sample of config 3: prune+compress of the full W, then the dense masked fp32 product for the
-    first 1024 rows of X."""
+    """The oracle (pure-PyTorch port of the reference semantics) on the host cores, on config 3 itself:
+    prune+compress and transposable mask of W, then both dense masked fp32 products once."""
     import oracle
     torch.set_num_threads(threads)
     gen = torch.Generator().manual_seed(3)
-    K, Nw, rows = 4096, 11008, 1024
-    X = torch.randn(rows, K, generator=gen).half()
+    M, K, Nw = 8192, 4096, 11008
+    X = torch.randn(M, K, generator=gen).half()
     W = (0.02 * torch.randn(Nw, K, generator=gen)).half()
+    dY = torch.randn(M, Nw, generator=gen).half()
     t0 = time.perf_counter()
     mask = oracle.prune24_mask(W)
     oracle.compress24(W, mask=mask)
     t_conv = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    w_t, _ = oracle.transposable_mask(W)
+    t_tr = time.perf_counter() - t0
     Wm = torch.where(mask, W, torch.zeros_like(W))
     oracle.spmm_ref(X[:64], Wm)
     t0 = time.perf_counter()
     oracle.spmm_ref(X, Wm)
+    oracle.spmm_ref(dY, w_t.t().contiguous())
     t_mm = time.perf_counter() - t0
-    tflops = 2.0 * rows * Nw * K / t_mm / 1e12
-    conv_gbps = 3.125 * Nw * K / t_conv / 1e9
+    tflops = 2 * 2.0 * M * Nw * K / t_mm / 1e12
     return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"oracle.spmm_ref fp32 on X[:{rows}] x masked W[{Nw},{K}] ({t_mm:.2f} s); "
-                      f"oracle prune+compress of the full W took {t_conv:.2f} s = {conv_gbps:.2f} GB/s algorithmic"}
+            "sample": f"the whole of config 3 once: oracle.spmm_ref fp32 forward + transposed ({t_mm:.2f} s); "
+                      f"oracle prune+compress of W {t_conv:.2f} s ({3.125 * Nw * K / t_conv / 1e9:.2f} GB/s algorithmic), "
+                      f"oracle transposable mask of W {t_tr:.2f} s ({5.0 * Nw * K / t_tr / 1e9:.2f} GB/s algorithmic)"}
 
 
 def main():
@@ -227,7 +234,8 @@ def main():
                    "M": M, "K": K, "N": Nw, "seed": 3},
         "roofline": {"bound": "mfma", "kernel": "spmm (SMFMAC)", "achieved": round(executed_tflops, 2),
                      "peak": MFMA_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(executed_tflops / MFMA_DENSE_PEAK_TFLOPS, 4),
-                     "traffic": None,
+                     "traffic": SPMM_TRAFFIC_BYTES,
+                     "algorithmic_bytes": 2 * (M * K + Nw * K // 2 + Nw * K // 16 + M * Nw),
                      "note": "achieved = executed flops (M*N*K, half the dense-equivalent 2MNK) per launch / HIP-event "
                              "launch time; SMFMAC executes MACs at the dense MFMA rate, so frac also equals "
                              "dense-equivalent rate / (2 x dense peak)",
