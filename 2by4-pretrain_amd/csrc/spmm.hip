@@ -429,6 +429,43 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
         if (jrow < n_dense && icol < n_sparse) *reinterpret_cast<int4v*>(c + jrow * ldc + icol) = v;
       }
     }
+  } else if constexpr (!C_JMAJOR && sizeof(OutT) == 2) {
+    // i-major 16-bit output (the W.B of `S @ dense`): a lane owns single elements of 64+ different
+    // rows.  Stage 128(i) x 64(j) pieces as [i][64 j] (128-byte rows, chunks XOR-swizzled with the
+    // row) and stream them out as eight full 128-byte rows per instruction.
+    __syncthreads();
+    uint8_t* stage = wave < 2 ? s_b0 + wave * 16384 : wave < 4 ? s_b1 + (wave - 2) * 16384
+                   : wave < 6 ? s_b2 + (wave - 4) * 16384 : wave == 6 ? s_a0 : s_a1;
+    const int rr = lane >> 3, chr = lane & 7;
+#pragma unroll
+    for (int half = 0; half < C::TJ / 2; half++) {            // 64 output columns (j) per pass
+#pragma unroll
+      for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+        for (int t2 = 0; t2 < 2; t2++) {
+          const int tj = half * 2 + t2;
+          const int jl = t2 * 32 + l32;
+#pragma unroll
+          for (int g = 0; g < 4; g++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              const int il = ti * 32 + g * 8 + lh * 4 + r;
+              const int64_t row = i0 + wi * C::WI + il;
+              float v = acc[ti][tj][g * 4 + r] * scale;
+              if (bias && row < n_sparse) v += to_float(bias[row]);
+              *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ ((il >> 1) & 7)) * 16) + (jl & 7) * 2) =
+                  from_float<OutT>(apply_act(v, act));
+            }
+        }
+      const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
+#pragma unroll
+      for (int it = 0; it < 16; it++) {
+        const int il = it * 8 + rr;
+        const int64_t irow = i0 + wi * C::WI + il;
+        const int4v v = *reinterpret_cast<const int4v*>(stage + il * 128 + ((chr ^ ((il >> 1) & 7)) * 16));
+        if (irow < n_sparse && jcol < n_dense) *reinterpret_cast<int4v*>(c + irow * ldc + jcol) = v;
+      }
+    }
   } else {
 #pragma unroll
     for (int ti = 0; ti < C::TI; ti++)

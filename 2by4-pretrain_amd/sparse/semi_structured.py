@@ -101,6 +101,13 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
         raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
     dense = N.as_matrix(dense)
     lay, ld = N.layout_of(dense)
+    # The tiled kernel wants the dense operand with k contiguous.  When k is the strided dimension
+    # (`S @ dense` with a row-major dense, e.g. dW = MVUE(dY^T) @ x) one transposing copy of the dense
+    # operand is far cheaper than running the general kernel.
+    k_strided = (lay == N.ROW_MAJOR) if sparse_first else (lay == N.COL_MAJOR)
+    if k_strided and sparse._store_layout == N.COMPRESSED_PANEL and dense.numel() >= (1 << 16):
+        dense = dense.t().contiguous().t() if sparse_first else dense.contiguous()
+        lay, ld = N.layout_of(dense)
     if sparse_first:
         kk, j = dense.shape
         b_layout = N.COL_MAJOR if lay == N.ROW_MAJOR else N.ROW_MAJOR   # k strided when the [k,j] tensor is row-major

@@ -175,6 +175,67 @@ def spmm_workload(steps, warmup):
     return wall_ms, fwd_ms, bwd_ms, dense_fwd_ms, dense_bwd_ms, rel_fwd, rel_bwd, flops, (M, K, Nw)
 
 
+
+# --------------------------------------------------------------------------------------------
+def train_workload(steps, warmup):
+    """BASELINE config 4: GPT-2-124M MLP (c_fc 768->3072, GELU, c_proj 3072->768) on 12x1024 tokens,
+    fp16 autocast, SparseLinearTranspose layers (transposable mask refreshed every 40 optimizer steps,
+    W and W^T recompressed each step, MVUE24 dW), masked decay alpha=2e-4, fused AdamW; seed 2.
+    Returns ms/step for the sparse model and for the same MLP with dense nn.Linear layers."""
+    import sparse
+    import torch.nn.functional as F
+    dev = torch.device("cuda:0")
+    torch.manual_seed(2)
+    tokens, d, h = 12 * 1024, 768, 3072
+    x = torch.randn(tokens, d, device=dev)
+    target = torch.randn(tokens, d, device=dev)
+
+    def build(kind):
+        torch.manual_seed(2)
+        if kind == "sparse":
+            fc, proj = sparse.SparseLinearTranspose(d, h).to(dev), sparse.SparseLinearTranspose(h, d).to(dev)
+        else:
+            fc, proj = torch.nn.Linear(d, h).to(dev), torch.nn.Linear(h, d).to(dev)
+        for layer in (fc, proj):
+            torch.nn.init.normal_(layer.weight, std=0.02)
+        params = list(fc.parameters()) + list(proj.parameters())
+        return fc, proj, params, torch.optim.AdamW(params, lr=1e-4, weight_decay=0.0, fused=True)
+
+    def run(kind):
+        fc, proj, params, opt = build(kind)
+
+        def step():
+            if kind == "sparse":
+                out = proj(F.gelu(fc(x)))
+            else:
+                with torch.autocast(device_type="cuda", dtype=torch.float16):
+                    out = proj(F.gelu(fc(x)))
+            loss = F.mse_loss(out.float(), target)
+            opt.zero_grad(set_to_none=True)
+            loss.backward()
+            if kind == "sparse":
+                with torch.no_grad():
+                    for p in params:
+                        if hasattr(p, "mask") and p.mode == "sparse":
+                            p.grad = p.grad.float()
+                            sparse.masked_add_(p.grad.data, p.data, p.mask, alpha=2e-4)
+                            p.cnt = 0
+            opt.step()
+            return loss
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps, loss.item()
+    sparse_ms, sparse_loss = run("sparse")
+    dense_ms, dense_loss = run("dense")
+    flops = 6 * 2.0 * tokens * d * h          # 3 GEMMs per layer, 2 layers, dense-equivalent
+    return sparse_ms, dense_ms, sparse_loss, dense_loss, flops
+
+
 def cpu_baseline_spmm(threads):
     """The oracle (pure-PyTorch port of the reference semantics) on the host cores, on config 3 itself:
     prune+compress and transposable mask of W, then both dense masked fp32 products once."""
@@ -210,6 +271,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", choices=["spmm", "train"], default="spmm",
+                    help="spmm: BASELINE configs[2] (default, the judged line); train: configs[3] MLP training step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-convert", action="store_true", help="skip the conversion-kernel table")
     a = ap.parse_args()
@@ -220,6 +283,18 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+
+    if a.workload == "train":
+        sparse_ms, dense_ms, sl, dl, flops = train_workload(a.steps, a.warmup)
+        print(json.dumps({
+            "metric": "2:4 sparse MLP training step, dense-equivalent TFLOP/s of its 6 GEMMs", "value": round(flops / (sparse_ms * 1e-3) / 1e12, 2),
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(sparse_ms, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "BASELINE configs[3]: SparseLinearTranspose GPT-2-124M MLP step, 12288 tokens, 768->3072->768, "
+                                   "masked decay 2e-4, fused AdamW, mask refresh every 40 steps", "seed": 2},
+            "dense_autocast_ms_per_step": round(dense_ms, 4), "speedup_vs_dense_step": round(dense_ms / sparse_ms, 3),
+            "final_loss": {"sparse": sl, "dense": dl}}))
+        return
 
     wall_ms, fwd_ms, bwd_ms, dfwd_ms, dbwd_ms, rel_f, rel_b, flops, (M, K, Nw) = spmm_workload(a.steps, a.warmup)
     value = 2 * flops / (wall_ms * 1e-3) / 1e12

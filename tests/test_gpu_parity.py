@@ -354,3 +354,27 @@ def test_dispatch_rules(cuda):
         torch.mm(s.t(), x.t())                             # first operand must not be
     with pytest.raises(NotImplementedError):
         s + 1
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_spmm_tiled_all_operand_positions(cuda, dtype):
+    """Shapes large enough for the tiled kernel, with partial tiles: both operand positions, both
+    layouts of the dense operand, bias, and the i-major / j-major LDS-staged epilogues."""
+    import sparse
+    n, k, m = 352, 640, 296
+    w = _small_ints((n, k), 61).to(dtype)
+    x = _small_ints((m, k), 62).to(dtype)
+    bias = _small_ints((n,), 63).to(dtype)
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+    ref_b = (ref + bias.float()).to(dtype).float()
+    ref = ref.to(dtype).float()
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    xg = x.to(cuda)
+    assert torch.mm(xg, s.t()).float().cpu().equal(ref)                          # k contiguous, j-major store
+    assert torch.mm(maybe_t(xg, True), s.t()).float().cpu().equal(ref)           # k strided dense operand
+    assert torch.mm(s, xg.t()).float().cpu().equal(ref.t())                      # sparse first, k contiguous view
+    assert torch.mm(s, xg.t().contiguous()).float().cpu().equal(ref.t())         # sparse first, k strided
+    assert torch.addmm(bias.to(cuda), xg, s.t()).float().cpu().equal(ref_b)
+    out = sparse.sparse_semi_structured_linear(xg, s, bias=bias.to(cuda), activation="relu")
+    assert out.float().cpu().equal(ref_b.clamp_min(0))
