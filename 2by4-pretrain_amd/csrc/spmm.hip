@@ -229,7 +229,7 @@ __global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
           OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act,
-          int tiles_i, int tiles_j) {
+          int tiles_i, int tiles_j, int splits, float* __restrict__ partial) {
   constexpr int ES = sizeof(T);
   constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
   constexpr int M_STEP = M_ROW / C::STEPS;
@@ -246,12 +246,15 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   __shared__ __attribute__((aligned(1024))) uint8_t s_m1[M_STAGE];
   __shared__ __attribute__((aligned(1024))) uint8_t s_m2[M_STAGE];
 
-  // ---- XCD-aware tile assignment
+  // ---- XCD-aware work assignment.  A unit of work is (k-split, tile); units are ordered split-major
+  // so that the units resident on an XCD belong to the same k range and share operand rows in L2.
   const int ntiles = tiles_i * tiles_j;
-  const int per_xcd = (ntiles + 7) / 8;
+  const int nunits = ntiles * splits;
+  const int per_xcd = (nunits + 7) / 8;
   const int bid = blockIdx.x;
-  const int tile = (bid & 7) * per_xcd + (bid >> 3);
-  if (tile >= ntiles) return;
+  const int unit = (bid & 7) * per_xcd + (bid >> 3);
+  if (unit >= nunits) return;
+  const int split = unit / ntiles, tile = unit - split * ntiles;
   constexpr int GH = C::GH;
   const int group = tile / (GH * tiles_j);
   const int gh = min(GH, tiles_i - group * GH);
@@ -264,9 +267,11 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wi = wave / C::WAVES_J, wj = wave % C::WAVES_J;
   const int l32 = lane & 31, lh = lane >> 5;
-  const int nstages = (int)((k * ES) / C::KB);
+  const int nstages_total = (int)((k * ES) / C::KB);
+  const int st_begin = (int)((int64_t)split * nstages_total / splits);
+  const int nstages = (int)((int64_t)(split + 1) * nstages_total / splits) - st_begin;
 
-  // ---- per-lane global sources of the copies (stage 0); LDS destinations are wave-uniform.
+  // ---- per-lane global sources of the copies (first stage of this unit); LDS destinations are wave-uniform.
   // B: copy q of a wave brings 8 rows x 128 bytes; lane -> (row, swizzled chunk).
   // A: stage st of rows i0..i0+255 is one contiguous run of 256*64 value bytes at (st*n_sparse + i0)*64
   //    (and 256*M_ROW metadata bytes): copy q brings 16 rows x 64 bytes.
@@ -276,20 +281,20 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   for (int q = 0; q < C::NB; q++) {
     const int row = (wave * C::NB + q) * 8 + (lane >> 3);
     const int ch = (lane & 7) ^ ((row >> 1) & 7);
-    gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16;
+    gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16 + (int64_t)st_begin * C::B_ROW;
   }
 #pragma unroll
   for (int q = 0; q < C::NA; q++) {
     const int row = (wave * C::NA + q) * 16 + (lane >> 2);
     const int ch = (lane & 3) ^ ((row >> 2) & 3);
-    ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16;
+    ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16 + (int64_t)st_begin * n_sparse * 64;
   }
   const bool has_meta_copy = wave < M_COPIES;
   const uint8_t* gm;
   {
     const int row = (wave % M_COPIES) * (1024 / M_ROW) + lane * 16 / M_ROW;
     // a 16-byte copy spans 16/M_ROW rows: clamp so that it never reaches past the last row
-    gm = a_meta + min(i0 + row, n_sparse - 16 / M_ROW) * M_ROW + (lane * 16) % M_ROW;
+    gm = a_meta + min(i0 + row, n_sparse - 16 / M_ROW) * M_ROW + (lane * 16) % M_ROW + (int64_t)st_begin * n_sparse * M_ROW;
   }
   const int64_t a_stage_stride = n_sparse * 64, m_stage_stride = n_sparse * M_ROW;
   constexpr int NCOPY = C::NB + C::NA + 1;       // copies per wave per stage (one less without metadata copy)
@@ -386,6 +391,23 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   }
   if (st < nstages) { pipe_step(st, s_a0, s_b0, s_m0, s_a2, s_b2, s_m2); st++; }
   if (st < nstages) { pipe_step(st, s_a1, s_b1, s_m1, s_a0, s_b0, s_m0); st++; }
+
+  // ---- split-K: park the float32 accumulators in the workspace, in register order (every group of
+  // four accumulators is one contiguous 16-byte-per-lane slab); spmm_reduce_splits finishes the job.
+  if (splits > 1) {
+    float* base = partial + (int64_t)unit * (C::BI * C::BJ);
+#pragma unroll
+    for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+      for (int tj = 0; tj < C::TJ; tj++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const int slab = (ti * C::TJ + tj) * 4 + g;
+          float4v v = {acc[ti][tj][g * 4], acc[ti][tj][g * 4 + 1], acc[ti][tj][g * 4 + 2], acc[ti][tj][g * 4 + 3]};
+          *reinterpret_cast<float4v*>(base + ((int64_t)slab * C::THREADS + tid) * 4) = v;
+        }
+    return;
+  }
 
   // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
   // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
@@ -494,18 +516,91 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   }
 }
 
+// Second pass of a split-K product: a block handles one eighth of a tile (the accumulator groups
+// `slab` of one ti), same lane -> element mapping as spmm_pipe; sums the `splits` float32 partial
+// tiles and applies scale / bias / activation / conversion.
+template <typename OutT, bool C_JMAJOR, typename C>
+__global__ void __launch_bounds__(C::THREADS)
+spmm_reduce_splits(const float* __restrict__ partial, int splits, int tiles_i, int tiles_j, int64_t n_sparse, int64_t n_dense,
+                   OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
+  const int ntiles = tiles_i * tiles_j;
+  const int tile = blockIdx.x;
+  constexpr int GH = C::GH;
+  const int group = tile / (GH * tiles_j);
+  const int gh = min(GH, tiles_i - group * GH);
+  const int in_group = tile - group * GH * tiles_j;
+  const int64_t i0 = (int64_t)(group * GH + in_group % gh) * C::BI, j0 = (int64_t)(in_group / gh) * C::BJ;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wi = wave / C::WAVES_J, wj = wave % C::WAVES_J;
+  const int l32 = lane & 31, lh = lane >> 5;
+  constexpr int NSLAB = C::TI * C::TJ * 4;
+  // gridDim.y blocks share the NSLAB accumulator groups of the tile
+  for (int slab = blockIdx.y; slab < NSLAB; slab += gridDim.y) {
+    const int ti = slab / (C::TJ * 4), tj = (slab / 4) % C::TJ, g = slab % 4;
+    float4v sum = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < splits; sp++) {
+      const float* base = partial + ((int64_t)sp * ntiles + tile) * (C::BI * C::BJ);
+      sum += *reinterpret_cast<const float4v*>(base + ((int64_t)slab * C::THREADS + tid) * 4);
+    }
+    const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
+    const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+    if (col >= n_dense || row >= n_sparse) continue;
+    OutT o[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      float v = sum[r] * scale;
+      if (bias) v += to_float(bias[row + r]);
+      o[r] = from_float<OutT>(apply_act(v, act));
+    }
+    if constexpr (C_JMAJOR) {
+      *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
+    }
+  }
+}
+
+// k-splits for shapes whose tiles cannot fill the 256 CUs (k-heavy products such as dW): as many as
+// fit, each at least 4 stages long, if the caller's workspace holds the float32 partial tiles.
+template <typename T, typename C>
+int choose_splits(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspace_bytes) {
+  const int64_t tiles = ((n_sparse + C::BI - 1) / C::BI) * ((n_dense + C::BJ - 1) / C::BJ);
+  const int64_t nstages = k * (int64_t)sizeof(T) / C::KB;
+  if (tiles >= 160) return 1;
+  int64_t splits = 256 / tiles;
+  if (splits > nstages / 4) splits = nstages / 4;
+  if (splits > 16) splits = 16;
+  while (splits > 1 && splits * tiles * C::BI * C::BJ * 4 > workspace_bytes) splits--;
+  return splits < 2 ? 1 : (int)splits;
+}
+
 template <typename T, typename OutT, typename C>
 int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
-                 int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
+                 int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
+                 void* workspace, int64_t workspace_bytes, hipStream_t s) {
   const int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI), tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
-  const int per_xcd = (tiles_i * tiles_j + 7) / 8;
+  const int splits = workspace ? choose_splits<T, C>(n_sparse, k, n_dense, workspace_bytes) : 1;
+  const int per_xcd = (tiles_i * tiles_j * splits + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
-  if (c_layout == TF24_COL_MAJOR)
+  const bool jm = c_layout == TF24_COL_MAJOR;
+  if (jm)
     hipLaunchKernelGGL((spmm_pipe<T, OutT, true, C>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
-                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
+                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j,
+                       splits, (float*)workspace);
   else
     hipLaunchKernelGGL((spmm_pipe<T, OutT, false, C>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
-                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j);
+                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j,
+                       splits, (float*)workspace);
+  if (splits > 1) {
+    dim3 rgrid((unsigned)(tiles_i * tiles_j), 8);
+    if (jm)
+      hipLaunchKernelGGL((spmm_reduce_splits<OutT, true, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
+                         n_sparse, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
+    else
+      hipLaunchKernelGGL((spmm_reduce_splits<OutT, false, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
+                         n_sparse, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
+  }
   return check_launch("tf24_spmm");
 }
 
@@ -528,12 +623,12 @@ int launch_general(const void* av, const void* am, bool panel, int64_t n_sparse,
 template <typename T>
 int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout,
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
-                 hipStream_t s) {
+                 void* workspace, int64_t workspace_bytes, hipStream_t s) {
   if (panel && b_layout == TF24_ROW_MAJOR && n_sparse >= 64 && n_dense >= 64) {
     switch (out_dtype) {
-      case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-      case TF24_BF16: return launch_tiled<T, bf16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-      case TF24_F32: return launch_tiled<T, float, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_BF16: return launch_tiled<T, bf16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_F32: return launch_tiled<T, float, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     }
   }
   switch (out_dtype) {
@@ -568,10 +663,21 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
   return TF24_OK;
 }
 
+extern "C" int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense) {
+  using namespace tf24;
+  const int64_t big = (int64_t)1 << 40;
+  int splits;
+  if (dtype == TF24_E4M3) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
+  else splits = choose_splits<f16_t, TiledCfg>(n_sparse, k, n_dense, big);
+  if (splits < 2) return 0;
+  const int64_t tiles = ((n_sparse + TiledCfg::BI - 1) / TiledCfg::BI) * ((n_dense + TiledCfg::BJ - 1) / TiledCfg::BJ);
+  return splits * tiles * TiledCfg::BI * TiledCfg::BJ * 4;
+}
+
 extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,
                          const void* b, int b_layout, int64_t ldb, int64_t n_dense,
                          void* c, int out_dtype, int c_layout, int64_t ldc,
-                         const void* bias, float scale, int activation, void* stream) {
+                         const void* bias, float scale, int activation, void* workspace, int64_t workspace_bytes, void* stream) {
   using namespace tf24;
   int rc = tf24_spmm_validate(dtype, n_sparse, k, b_layout, ldb, n_dense, out_dtype, c_layout, ldc, activation);
   if (rc) return rc;
@@ -580,8 +686,8 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout,
   const bool panel = a_layout == TF24_COMPRESSED_PANEL;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
-    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
   }
 }

@@ -40,7 +40,9 @@ _SIGNATURES = {
     "tf24_sparse24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _p, _p]),
     "tf24_mvue24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _i64, _p, _p]),
     "tf24_masked_add": (_i, [_p, _i, _p, _i, _p, _i, _i64, _f, _p]),
-    "tf24_spmm": (_i, [_p, _p, _i, _i, _i64, _i64, _p, _i, _i64, _i64, _p, _i, _i, _i64, _p, _f, _i, _p]),
+    "tf24_spmm": (_i, [_p, _p, _i, _i, _i64, _i64, _p, _i, _i64, _i64, _p, _i, _i, _i64, _p, _f, _i, _p, _i64, _p]),
+    "tf24_spmm_workspace_bytes": (_i64, [_i, _i64, _i64, _i64]),
+    "tf24_transpose": (_i, [_p, _i, _i64, _i64, _i64, _p, _i64, _p]),
     "tf24_spmm_validate": (_i, [_i, _i64, _i64, _i, _i64, _i64, _i, _i, _i64, _i]),
 }
 
@@ -117,3 +119,11 @@ def as_matrix(t, like=None):
 
 def ptr(t):
     return None if t is None else t.data_ptr()
+
+
+def transposed_copy(t):
+    """Row-major [cols, rows] copy of the 2-d row-major tensor t [rows, cols] (HIP tile transpose)."""
+    rows, cols = t.shape
+    out = torch.empty((cols, rows), dtype=t.dtype, device=t.device)
+    check(lib().tf24_transpose(t.data_ptr(), dtype_code(t.dtype), t.stride(0), rows, cols, out.data_ptr(), rows, stream_ptr()))
+    return out

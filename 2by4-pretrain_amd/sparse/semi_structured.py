@@ -106,7 +106,13 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     # operand is far cheaper than running the general kernel.
     k_strided = (lay == N.ROW_MAJOR) if sparse_first else (lay == N.COL_MAJOR)
     if k_strided and sparse._store_layout == N.COMPRESSED_PANEL and dense.numel() >= (1 << 16):
-        dense = dense.t().contiguous().t() if sparse_first else dense.contiguous()
+        v = 16 // dense.element_size()
+        row_major = dense if sparse_first else dense.t()          # the view that is row-major: [k, j]
+        if row_major.shape[0] % v == 0 and row_major.shape[1] % v == 0:
+            flipped = N.transposed_copy(row_major)                # [j, k], k contiguous
+        else:
+            flipped = row_major.t().contiguous()
+        dense = flipped.t() if sparse_first else flipped
         lay, ld = N.layout_of(dense)
     if sparse_first:
         kk, j = dense.shape
@@ -125,10 +131,12 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
         bias = bias.to(out_dtype).contiguous()
         if bias.numel() != n:
             raise RuntimeError(f"bias must have {n} elements, got {bias.numel()}")
+    ws_bytes = N.lib().tf24_spmm_workspace_bytes(N.dtype_code(values.dtype), n, k, j)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dense.device) if ws_bytes else None
     N.check(N.lib().tf24_spmm(
         values.data_ptr(), meta.data_ptr(), sparse._store_layout, N.dtype_code(values.dtype), n, k,
         dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.dtype_code(out_dtype), c_layout, out.stride(0),
-        N.ptr(bias), float(scale), activation, N.stream_ptr()))
+        N.ptr(bias), float(scale), activation, N.ptr(workspace), ws_bytes, N.stream_ptr()))
     return out
 
 

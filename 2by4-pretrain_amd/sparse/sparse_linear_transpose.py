@@ -28,10 +28,11 @@ class sparse_linear_transpose(autograd.Function):
         ctx.save_for_backward(input, weight_sparse_T, bias)
         ctx.shape = input.shape
         input = input.view(-1, input.shape[-1])
-        output = torch.mm(input, weight_sparse.t())
         if bias is None:
-            return output.view(*ctx.shape[:-1], -1)
-        return output.view(*ctx.shape[:-1], -1) + bias
+            output = torch.mm(input, weight_sparse.t())
+        else:
+            output = torch.addmm(bias, input, weight_sparse.t())      # bias added in the matmul epilogue
+        return output.view(*ctx.shape[:-1], -1)
 
     @staticmethod
     @custom_bwd(device_type="cuda")

@@ -158,13 +158,28 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  *              TF24_COL_MAJOR stores it at j*ldc + i ([n_dense,n_sparse]: the Y of X.W^T)
  *   bias       NULL or [n_sparse] of out_dtype's float family (added per sparse row i)
  *   scale      multiplies the accumulator before bias (1.0 for 16-bit; scale_a*scale_b for fp8)
+ *   workspace  NULL, or scratch of workspace_bytes for k-split partial tiles: products whose output
+ *              tiles cannot fill the GPU (k-heavy shapes such as dW) are split along k and reduced in
+ *              a second launch.  tf24_spmm_workspace_bytes() gives the size that enables every split
+ *              the heuristic would take (0 = the shape is never split).  Deterministic either way.
  * Shape rules (.cu:101-109): n_sparse % 32 == 0, k % 64 == 0 (16-bit) / 128 (8-bit),
  * n_dense % 8 == 0 (16-bit) / 16 (8-bit).
  */
 int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,
               const void* b, int b_layout, int64_t ldb, int64_t n_dense,
               void* c, int out_dtype, int c_layout, int64_t ldc,
-              const void* bias, float scale, int activation, void* stream);
+              const void* bias, float scale, int activation, void* workspace, int64_t workspace_bytes, void* stream);
+int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense);
+
+/*
+ * out[c, r] = in[r, c] for 2-byte (F16|BF16) and 1-byte (E4M3|U8) elements; in [rows, cols] with
+ * leading dimension ld_in, out [cols, rows] with ld_out.  No counterpart in the reference (CUTLASS
+ * reads either operand layout): it feeds tf24_spmm's fast kernel, which wants the dense operand
+ * with k contiguous, when `S @ dense` arrives with a row-major dense (dW = MVUE(dY^T) @ x).
+ * rows, cols and leading dimensions must be multiples of 16 bytes worth of elements.
+ */
+int tf24_transpose(const void* in, int dtype, int64_t ld_in, int64_t rows, int64_t cols, void* out, int64_t ld_out,
+                   void* stream);
 int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_layout, int64_t ldb, int64_t n_dense,
                        int out_dtype, int c_layout, int64_t ldc, int activation);
 

@@ -378,3 +378,40 @@ def test_spmm_tiled_all_operand_positions(cuda, dtype):
     assert torch.addmm(bias.to(cuda), xg, s.t()).float().cpu().equal(ref_b)
     out = sparse.sparse_semi_structured_linear(xg, s, bias=bias.to(cuda), activation="relu")
     assert out.float().cpu().equal(ref_b.clamp_min(0))
+
+
+@pytest.mark.parametrize("dims", [(256, 4096, 256), (96, 2048, 520), (352, 12288 // 4, 200)])
+def test_spmm_split_k_is_exact_and_deterministic(cuda, dims):
+    """k-heavy shapes whose tiles cannot fill the GPU take the split-K path (float32 partial tiles in a
+    workspace + reduction launch); small-integer operands keep every partial sum exact."""
+    import sparse
+    from sparse import _native as N
+    n, k, m = dims
+    assert N.lib().tf24_spmm_workspace_bytes(N.F16, n, k, m) > 0
+    w = _small_ints((n, k), 71, -2, 3).half()
+    x = _small_ints((m, k), 72, -2, 3).half()
+    bias = _small_ints((n,), 73).half()
+    mask = oracle.prune24_mask(w)
+    ref = oracle.spmm_ref(x, torch.where(mask, w, torch.zeros_like(w)))
+    s = sparse.to_sparse_semi_structured(w.to(cuda))
+    out = torch.mm(x.to(cuda), s.t())
+    assert out.float().cpu().equal(ref.half().float())
+    assert torch.mm(x.to(cuda), s.t()).equal(out)                                  # bit-reproducible
+    assert torch.mm(s, x.to(cuda).t().contiguous()).float().cpu().equal(ref.t().half().float())
+    outb = torch.addmm(bias.to(cuda), x.to(cuda), s.t())
+    assert outb.float().cpu().equal((ref + bias.float()).half().float())
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, torch.uint8])
+@pytest.mark.parametrize("shape", [(64, 64), (200, 136), (1024, 768), (48, 4096)])
+def test_transpose_copy(cuda, dtype, shape):
+    from sparse import _native as N
+    rows, cols = shape
+    if dtype == torch.uint8:
+        rows, cols = (rows + 15) // 16 * 16, (cols + 15) // 16 * 16
+        t = torch.randint(0, 255, (rows, cols), dtype=torch.uint8, generator=torch.Generator().manual_seed(81))
+    else:
+        t = randn((rows, cols), dtype, 81)
+    out = N.transposed_copy(t.to(cuda))
+    assert out.shape == (cols, rows) and out.is_contiguous()
+    assert_same(out, t.t().contiguous())
