@@ -13,7 +13,16 @@ enum { OP_SOFT = 0, OP_SPARSE24 = 1, OP_MVUE = 2 };
 template <int OP>
 __device__ __forceinline__ uint32_t group_op(const float (&x)[4], float r0, float r1, float (&y)[4]) {
   if constexpr (OP == OP_MVUE) {
-    return mvue4(x[0], x[1], x[2], x[3], r0, r1, y[0], y[1], y[2], y[3]);
+    // only the two kept values are rescaled; with fewer than two mask bits the kept element is
+    // still one of the two encoded positions
+    const Mvue4 g = mvue4(x[0], x[1], x[2], x[3], r0, r1);
+    const uint32_t nib = encode_nibble(g.mask);
+    const uint32_t pa = nib & 3, pb = nib >> 2;
+    const float ya = mvue_rescale(select4(pa, x[0], x[1], x[2], x[3]), select4(pa, g.p[0], g.p[1], g.p[2], g.p[3]), g.in_range);
+    const float yb = mvue_rescale(select4(pb, x[0], x[1], x[2], x[3]), select4(pb, g.p[0], g.p[1], g.p[2], g.p[3]), g.in_range);
+#pragma unroll
+    for (int i = 0; i < 4; i++) y[i] = (uint32_t)i == pa ? ya : yb;
+    return g.mask;
   } else {
     uint32_t mb = magnitude_mask4(x[0], x[1], x[2], x[3]);
     if constexpr (OP == OP_SOFT) {

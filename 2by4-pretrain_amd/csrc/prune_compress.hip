@@ -15,20 +15,29 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kUnroll = 4;
 
+// Kept-mask bits of one group; in MVUE mode also the inclusion probabilities the two kept
+// values are divided by.
 template <typename In, int MODE, typename MaskT>
-__device__ __forceinline__ uint32_t prune_group(const float (&x)[4], const MaskT* mk, float r0, float r1, float (&y)[4]) {
+__device__ __forceinline__ uint32_t prune_group(const float (&x)[4], const MaskT* mk, float r0, float r1, Mvue4& g) {
   if constexpr (MODE == TF24_PRUNE_MAGNITUDE) {
-    y[0] = x[0]; y[1] = x[1]; y[2] = x[2]; y[3] = x[3];
     return magnitude_mask4(x[0], x[1], x[2], x[3]);
   } else if constexpr (MODE == TF24_PRUNE_MASK) {
-    y[0] = x[0]; y[1] = x[1]; y[2] = x[2]; y[3] = x[3];
     uint32_t b = 0;
 #pragma unroll
     for (int i = 0; i < 4; i++) b |= (uint32_t)(to_float(mk[i]) != 0.0f) << i;
     return b;
   } else {
-    return mvue4(x[0], x[1], x[2], x[3], r0, r1, y[0], y[1], y[2], y[3]);
+    g = mvue4(x[0], x[1], x[2], x[3], r0, r1);
+    return g.mask;
   }
+}
+
+// The value stored for metadata position pos (0..3) of a group.
+template <int MODE>
+__device__ __forceinline__ float kept_value(uint32_t pos, const float (&x)[4], const Mvue4& g) {
+  float v = select4(pos, x[0], x[1], x[2], x[3]);
+  if constexpr (MODE == TF24_PRUNE_MVUE) v = mvue_rescale(v, select4(pos, g.p[0], g.p[1], g.p[2], g.p[3]), g.in_range);
+  return v;
 }
 
 // ------------------------------------------------------------------ row-major
@@ -85,13 +94,14 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       }
 #pragma unroll
       for (int g = 0; g < 2; g++) {
-        float x[4], y[4];
+        float x[4];
+        Mvue4 pr;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = to_float(in.v[4 * g + i]);
-        uint32_t mb = prune_group<In, MODE, MaskT>(x, &mk.v[4 * g], r[2 * g], r[2 * g + 1], y);
+        uint32_t mb = prune_group<In, MODE, MaskT>(x, &mk.v[4 * g], r[2 * g], r[2 * g + 1], pr);
         uint32_t nib = encode_nibble(mb);
-        out.v[2 * g] = from_float<Out>(select4(nib & 3, y[0], y[1], y[2], y[3]));
-        out.v[2 * g + 1] = from_float<Out>(select4(nib >> 2, y[0], y[1], y[2], y[3]));
+        out.v[2 * g] = from_float<Out>(kept_value<MODE>(nib & 3, x, pr));
+        out.v[2 * g + 1] = from_float<Out>(kept_value<MODE>(nib >> 2, x, pr));
         mbyte |= nib << (4 * g);
       }
       out.store(values + ounit * 4);
@@ -141,17 +151,18 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     }
 #pragma unroll
     for (int i = 0; i < R; i++) {
-      float x[4], y[4];
+      float x[4];
+      Mvue4 pr;
       MaskT mrow[4];
 #pragma unroll
       for (int c = 0; c < 4; c++) { x[c] = to_float(in[c].v[i]); if constexpr (MODE == TF24_PRUNE_MASK) mrow[c] = mk[c].v[i]; }
       float u0 = 0.f, u1 = 0.f;
       if constexpr (MODE == TF24_PRUNE_MVUE) { u0 = rr[0].v[i]; u1 = rr[1].v[i]; }
-      uint32_t mb = prune_group<In, MODE, MaskT>(x, mrow, u0, u1, y);
+      uint32_t mb = prune_group<In, MODE, MaskT>(x, mrow, u0, u1, pr);
       uint32_t nib = encode_nibble(mb);
       Pack<Out, 2> o;
-      o.v[0] = from_float<Out>(select4(nib & 3, y[0], y[1], y[2], y[3]));
-      o.v[1] = from_float<Out>(select4(nib >> 2, y[0], y[1], y[2], y[3]));
+      o.v[0] = from_float<Out>(kept_value<MODE>(nib & 3, x, pr));
+      o.v[1] = from_float<Out>(kept_value<MODE>(nib >> 2, x, pr));
       const int lr = rchunk * R + i;
       o.store(reinterpret_cast<Out*>(s_val + lr * VPITCH) + grp * 2);
       // two groups share a metadata byte: even group low nibble, odd group high nibble

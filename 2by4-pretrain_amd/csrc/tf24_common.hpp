@@ -136,20 +136,58 @@ __device__ __forceinline__ T select4(uint32_t pos, T v0, T v1, T v2, T v3) {
   return (pos & 2) ? hi : lo;
 }
 
-// MVUE24 of one group in float32, in the reference's operation order (no contraction).
-// Outputs the rescaled values y_i = x_i / p_i and the kept-mask bits.
-__device__ __forceinline__ uint32_t mvue4(float x0, float x1, float x2, float x3, float r0, float r1,
-                                          float& y0, float& y1, float& y2, float& y3) {
+// Float32 division for operands inside the normal range.  This is the arithmetic the compiler's
+// own division performs between its v_div_scale and v_div_fixup steps: one Newton step on
+// v_rcp_f32, then two residual corrections of the quotient.  It returns the correctly rounded
+// quotient whenever v_div_scale would leave both operands unscaled and v_div_fixup would pass the
+// result through: numerator and denominator finite, non-zero and normal, |numerator| > 2^-104,
+// denominator < 2^126, exponent difference below 96 and a normal quotient.  Callers establish those
+// bounds and use operator/ outside them.  A reciprocal can be shared between quotients.
+__device__ __forceinline__ float refined_rcp(float b) {
+  float r = __builtin_amdgcn_rcpf(b);
+  return __builtin_fmaf(__builtin_fmaf(-b, r, 1.0f), r, r);
+}
+__device__ __forceinline__ float div_in_range(float a, float b, float r) {
+  float q = a * r;
+  q = __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
+  return __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
+}
+
+// MVUE24 of one group in float32, in the reference's operation order (no contraction): inclusion
+// probabilities p_i and the kept-mask bits.  The kept values are x_i / p_i (mvue_rescale); only
+// the two kept ones need the division.
+//
+// in_range: |x_i| + eps >= 2^-23 always, so with sum < 2^40 and every s_i = sum - a_i > 0 (then
+// s_i >= 2^-46) the quotients t_i = a_i/sum >= 2^-63 and k_i = t_i/s_i >= 2^-104 meet the bounds of
+// div_in_range; p_i >= t_i because k >= k_i for a rounded sum of non-negatives.
+struct Mvue4 {
+  float p[4];
+  uint32_t mask;
+  bool in_range;
+};
+
+__device__ __forceinline__ Mvue4 mvue4(float x0, float x1, float x2, float x3, float r0, float r1) {
   const float eps = 1.19209e-07f;
   float a0 = __builtin_fabsf(x0) + eps, a1 = __builtin_fabsf(x1) + eps;
   float a2 = __builtin_fabsf(x2) + eps, a3 = __builtin_fabsf(x3) + eps;
   float sum = ((a0 + a1) + a2) + a3;
-  float t0 = a0 / sum, t1 = a1 / sum, t2 = a2 / sum, t3 = a3 / sum;
   float s0 = sum - a0, s1 = sum - a1, s2 = sum - a2, s3 = sum - a3;
-  float k0 = t0 / s0, k1 = t1 / s1, k2 = t2 / s2, k3 = t3 / s3;
+  Mvue4 g;
+  g.in_range = (sum < 0x1p40f) & (s0 > 0.0f) & (s1 > 0.0f) & (s2 > 0.0f) & (s3 > 0.0f);
+  float t0, t1, t2, t3, k0, k1, k2, k3;
+  if (g.in_range) {
+    const float rs = refined_rcp(sum);
+    t0 = div_in_range(a0, sum, rs); t1 = div_in_range(a1, sum, rs);
+    t2 = div_in_range(a2, sum, rs); t3 = div_in_range(a3, sum, rs);
+    k0 = div_in_range(t0, s0, refined_rcp(s0)); k1 = div_in_range(t1, s1, refined_rcp(s1));
+    k2 = div_in_range(t2, s2, refined_rcp(s2)); k3 = div_in_range(t3, s3, refined_rcp(s3));
+  } else {
+    t0 = a0 / sum; t1 = a1 / sum; t2 = a2 / sum; t3 = a3 / sum;
+    k0 = t0 / s0; k1 = t1 / s1; k2 = t2 / s2; k3 = t3 / s3;
+  }
   float k = ((k0 + k1) + k2) + k3;
-  float p0 = t0 + a0 * (k - k0), p1 = t1 + a1 * (k - k1);
-  float p2 = t2 + a2 * (k - k2), p3 = t3 + a3 * (k - k3);
+  g.p[0] = t0 + a0 * (k - k0); g.p[1] = t1 + a1 * (k - k1);
+  g.p[2] = t2 + a2 * (k - k2); g.p[3] = t3 + a3 * (k - k3);
   bool m0 = r0 <= t0;
   bool m1 = (r0 <= (t0 + t1)) & !m0;
   bool m2 = (r0 <= ((t0 + t1) + t2)) & !m1 & !m0;
@@ -161,8 +199,20 @@ __device__ __forceinline__ uint32_t mvue4(float x0, float x1, float x2, float x3
   bool e1 = (t <= (d0 + d1)) & !e0;
   bool e2 = (t <= ((d0 + d1) + d2)) & !e1 & !e0;
   bool e3 = !e2 & !e1 & !e0;
-  y0 = x0 / p0; y1 = x1 / p1; y2 = x2 / p2; y3 = x3 / p3;
-  return (uint32_t)(m0 | e0) | ((uint32_t)(m1 | e1) << 1) | ((uint32_t)(m2 | e2) << 2) | ((uint32_t)(m3 | e3) << 3);
+  g.mask = (uint32_t)(m0 | e0) | ((uint32_t)(m1 | e1) << 1) | ((uint32_t)(m2 | e2) << 2) | ((uint32_t)(m3 | e3) << 3);
+  return g;
+}
+
+// x / p for a value of a group whose probabilities came from mvue4.  In range: p in [2^-63, 2],
+// |x| <= sum * p (so the exponent difference stays below 96) and |x| >= 2^-100 keeps the quotient
+// normal; a zero numerator returns the signed zero the division would.
+__device__ __forceinline__ float mvue_rescale(float x, float p, bool in_range) {
+  const bool ok = in_range & (p <= 2.0f) & ((x == 0.0f) | (__builtin_fabsf(x) >= 0x1p-100f));
+  if (ok) {
+    float q = div_in_range(x, p, refined_rcp(p));
+    return x == 0.0f ? x : q;
+  }
+  return x / p;
 }
 
 }  // namespace tf24

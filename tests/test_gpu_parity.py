@@ -157,6 +157,40 @@ def test_mvue_compress(cuda, shape, in_dtype, out_dtype, col_major):
     assert_same(s.indices(), want_m, "meta")
 
 
+def _wide_range(shape, seed):
+    """float32 values whose exponents span denormals to 2^60, with zeros, negative zeros and groups
+    dominated by one element (sum - a_i rounds to zero): operands the in-range division must hand
+    to the general one."""
+    g = torch.Generator().manual_seed(seed)
+    expo = torch.randint(-140, 61, shape, generator=g).float()
+    w = torch.randn(shape, generator=g) * torch.exp2(expo)
+    flat = w.view(-1, 4)
+    flat[0::7, 1] = 0.0
+    flat[3::7, 2] = -0.0
+    flat[5::11] = torch.tensor([1.0e6, 1.0e-7, 0.0, -1.0e-7])
+    flat[6::13] = torch.tensor([3.0e38, 1.0, -2.0e38, 1.0e-30])
+    return w
+
+
+@pytest.mark.parametrize("col_major", [False, True])
+def test_mvue_wide_dynamic_range(cuda, col_major):
+    import sparse
+    w = _wide_range((64, 256), 18)
+    u = torch.rand(w.shape, generator=torch.Generator().manual_seed(19))
+    want = oracle.mvue24_dense(w, u)
+    got = sparse.MVUE24_approx_triton(maybe_t(w.to(cuda), col_major), rand=maybe_t(u.to(cuda), col_major)).cpu()
+    assert torch.equal(got.isnan(), want.isnan())
+    ok = ~want.isnan()
+    assert_same(torch.where(ok, got, torch.zeros(())), torch.where(ok, want, torch.zeros(())), "mvue dense, wide range")
+    want_v, want_m, _ = oracle.mvue24(w, u, out_dtype=BF16)
+    s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major), MVUE24=True, rand=maybe_t(u.to(cuda), col_major), dtype=BF16)
+    assert_same(s.indices(), want_m, "meta")
+    gv = s.values().cpu()
+    assert torch.equal(gv.isnan(), want_v.isnan())
+    okv = ~want_v.isnan()
+    assert_same(torch.where(okv, gv, torch.zeros((), dtype=BF16)), torch.where(okv, want_v, torch.zeros((), dtype=BF16)), "values, wide range")
+
+
 def test_mvue_default_rand_keeps_two(cuda):
     import sparse
     w = randn((64, 128), F16, 17).to(cuda)
