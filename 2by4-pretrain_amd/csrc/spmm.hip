@@ -150,22 +150,24 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 // ------------------------------------------------------------------------------------------
 // Tiled kernel: A in the panel layout, B with k contiguous.
 //
-// A block computes a 256(i) x 256(j) tile with V_SMFMAC_F32_32X32X32_{F16,BF16} / 32X32X64_FP8.
-// Two wave arrangements (template parameter Cfg):
-//   Cfg8: 8 waves (2 along i x 4 along j), wave tile 128 x 64 = 4 x 2 instructions, 2 waves per SIMD
-//   Cfg4: 4 waves (2 x 2), wave tile 128 x 128 = 4 x 4 instructions, 256 accumulator registers,
-//         1 wave per SIMD: fewer LDS reads per instruction, but measured slower (kept for reference)
+// A block computes a 256(i) x 256(j) tile with V_SMFMAC_F32_32X32X32_{F16,BF16} / 32X32X64_FP8:
+// 8 waves (2 along i x 4 along j), wave tile 128 x 64 = 4 x 2 instructions, 2 waves per SIMD.
+// (4 waves with 128 x 128 wave tiles and 256 accumulators read less LDS per instruction but were
+// measured slower: with one wave per SIMD nothing covers a wave's own stalls.)
 // Operands go global -> LDS directly (GLOBAL_LOAD_LDS_DWORDX4: lane l of a wave writes
 // LDS[base + 16*l], a wave fills 1 KB of contiguous LDS) through a ring of three stage buffers of
 // 128 bytes of dense k per row (two instruction steps): while stage s is multiplied, the copies of
 // stages s+1 and s+2 are in flight.  LDS rows are unpadded; bank conflicts are avoided by
 // XOR-swizzling the 16-byte chunk index with row bits (B: chunk ^ ((row>>1)&7) in 128-byte rows,
 // A: chunk ^ ((row>>2)&3) in 64-byte rows), applied on the global side of the copy and again in the
-// fragment reads.  The three buffers are separate LDS objects and the stage loop is unrolled by
-// three, so that every LDS access names its buffer statically.
+// fragment reads.  The three buffers are slices of one LDS array addressed by a rotating
+// wave-uniform offset; the copies are written in assembly the compiler does not look into, so the
+// only LDS accesses it sees in the main loop are fragment reads.
 // Workgroup ids are remapped so that the 8 XCDs (ids are dealt round-robin) each walk a
 // contiguous range of tiles in an 8-tile-high grouped raster: the ~32 tiles resident on an XCD
 // form an 8 x 4 patch that shares A rows and B columns in that XCD's L2.
+// At sustained clocks this kernel runs against the board's power limit (the shader clock settles
+// near 2.1 GHz of 2.4): what buys time is fewer bytes moved per instruction, not a tighter schedule.
 // ------------------------------------------------------------------------------------------
 template <typename T> struct mma32;
 template <> struct mma32<f16_t> {
@@ -201,9 +203,7 @@ struct TileCfgT {
   static constexpr int NB = BJ * B_ROW / 1024 / NW;   // 1 KB copies per wave per stage: B
   static constexpr int NA = BI * A_ROW / 1024 / NW;   //                                 A values
 };
-using Cfg8 = TileCfgT<4, 2>;
-using Cfg4 = TileCfgT<2, 4>;
-using TiledCfg = Cfg8;
+using TiledCfg = TileCfgT<4, 2>;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -235,16 +235,10 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   constexpr int M_STEP = M_ROW / C::STEPS;
   constexpr int M_COPIES = C::BI * M_ROW / 1024;            // 1 KB copies per stage: metadata (2 or 4)
   static_assert(M_COPIES <= C::NW, "one metadata copy per wave at most");
+  // one stage buffer = [A values | B | A metadata]; three of them rotate
   constexpr int A_STAGE = C::BI * C::A_ROW, B_STAGE = C::BJ * C::B_ROW, M_STAGE = C::BI * M_ROW;
-  __shared__ __attribute__((aligned(1024))) uint8_t s_a0[A_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_a1[A_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_a2[A_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_b0[B_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_b1[B_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_b2[B_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_m0[M_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_m1[M_STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t s_m2[M_STAGE];
+  constexpr int B_AT = A_STAGE, M_AT = A_STAGE + B_STAGE, STAGE_BYTES = A_STAGE + B_STAGE + M_STAGE;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[3 * STAGE_BYTES];
 
   // ---- XCD-aware work assignment.  A unit of work is (k-split, tile); units are ordered split-major
   // so that the units resident on an XCD belong to the same k range and share operand rows in L2.
@@ -299,14 +293,16 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   const int64_t a_stage_stride = n_sparse * 64, m_stage_stride = n_sparse * M_ROW;
   constexpr int NCOPY = C::NB + C::NA + 1;       // copies per wave per stage (one less without metadata copy)
 
-  auto issue_one = [&](int q, int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
-    if (q < C::NB) g2l16(gb[q] + (int64_t)st * C::B_ROW, lds_offset(sb) + (wave * C::NB + q) * 1024);
-    else if (q < C::NB + C::NA) g2l16(ga[q - C::NB] + (int64_t)st * a_stage_stride, lds_offset(sa) + (wave * C::NA + q - C::NB) * 1024);
-    else if (has_meta_copy) g2l16(gm + (int64_t)st * m_stage_stride, lds_offset(sm) + wave * 1024);
+  // copy q of this wave for stage st into the stage buffer at LDS byte address `dst`
+  const uint32_t smem_at = lds_offset(smem);
+  auto issue_one = [&](int q, int st, uint32_t dst) {
+    if (q < C::NB) g2l16(gb[q] + (int64_t)st * C::B_ROW, dst + B_AT + (wave * C::NB + q) * 1024);
+    else if (q < C::NB + C::NA) g2l16(ga[q - C::NB] + (int64_t)st * a_stage_stride, dst + (wave * C::NA + q - C::NB) * 1024);
+    else if (has_meta_copy) g2l16(gm + (int64_t)st * m_stage_stride, dst + M_AT + wave * 1024);
   };
-  auto issue = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm) {
+  auto issue = [&](int st, uint32_t dst) {
 #pragma unroll
-    for (int q = 0; q < NCOPY; q++) issue_one(q, st, sa, sb, sm);
+    for (int q = 0; q < NCOPY; q++) issue_one(q, st, dst);
   };
 
   float16v acc[C::TI][C::TJ];
@@ -329,68 +325,105 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   }
   const int m_off = a_row * M_ROW + lh * (M_STEP / 2);
 
-  // ---- one stage: barrier (the stage's copies have landed and every wave is done with the buffer
-  // that is refilled next), then the two instruction steps.  The copies of stage+2 are spread
-  // between the matrix instructions: issued in a burst they would queue in the texture-address unit
-  // and hold back the fragment reads behind them.  (Double-buffering the fragments in registers
-  // across the barrier, and 128x128 wave tiles with one wave per SIMD, were both measured slower:
-  // the two waves of a SIMD already hide each other's LDS latency.)
-  auto compute = [&](const uint8_t* sa, const uint8_t* sb, const uint8_t* sm, bool copies, int pst, uint8_t* na, uint8_t* nb,
-                     uint8_t* nm) {
-#pragma unroll
-    for (int step = 0; step < C::STEPS; step++) {
-      int4v af[C::TI];
-      int idx[C::TI];
-      int8v bf[C::TJ];
-#pragma unroll
-      for (int ti = 0; ti < C::TI; ti++) {
-        af[ti] = *reinterpret_cast<const int4v*>(sa + a_off[step] + ti * 32 * C::A_ROW);
-        if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(sm + m_off + ti * 32 * M_ROW + step * M_STEP);
-        else idx[ti] = *reinterpret_cast<const int*>(sm + m_off + ti * 32 * M_ROW + step * M_STEP);
-      }
-#pragma unroll
-      for (int tj = 0; tj < C::TJ; tj++) {
-        const int4v lo = *reinterpret_cast<const int4v*>(sb + b_off[step][0] + tj * 32 * C::B_ROW);
-        const int4v hi = *reinterpret_cast<const int4v*>(sb + b_off[step][1] + tj * 32 * C::B_ROW);
-        bf[tj] = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      }
-#pragma unroll
-      for (int ti = 0; ti < C::TI; ti++) {
-#pragma unroll
-        for (int tj = 0; tj < C::TJ; tj++) acc[ti][tj] = mma32<T>::run(af[ti], bf[tj], acc[ti][tj], idx[ti]);
-        // one or two copies after each row of instructions
-        constexpr int PER_SLOT = (NCOPY + C::STEPS * C::TI - 1) / (C::STEPS * C::TI);
-#pragma unroll
-        for (int u = 0; u < PER_SLOT; u++) {
-          const int q = (step * C::TI + ti) * PER_SLOT + u;
-          if (q < NCOPY && copies) {
-            __builtin_amdgcn_sched_barrier(0);
-            issue_one(q, pst, na, nb, nm);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
-      }
+  // ---- main loop: a software pipeline over instruction steps.  While the matrix instructions of a
+  // step run from one register set, the fragments of the next step are read from LDS into the
+  // other, a few reads after every row of instructions: read in a block at the start of a step, the
+  // eight waves' requests fill the LDS queue, every wave stalls on issue, and the matrix pipes wait.
+  // The copies of the stage two ahead are spread over the same gaps (issued in a burst they would
+  // queue in the texture-address unit and hold back the fragment reads).
+  // One workgroup barrier per stage, B(s), placed before the first fragment read of stage s: every
+  // wave arrives having waited for its own copies of stage s and with all its reads of stage s-1
+  // complete, so behind B(s) stage s is visible and the buffer of stage s-1 is free for the copies
+  // of stage s+2.  The matrix instructions of the last step of stage s-1 are issued behind B(s),
+  // from registers, with the first reads of stage s between them.
+  int4v af[2][C::TI];
+  int idx[2][C::TI];
+  int4v bf[2][C::TJ][2];                         // the two 16-byte halves of a dense fragment
+  // The reads of a step, in the order the next step's instructions need them: its first row of
+  // instructions takes every dense fragment and sparse fragment 0, row r then only needs sparse
+  // fragment r.  Read n: dense half-fragment n (fragment n/2, half n%2) for n < 2*TJ, then sparse
+  // fragment and index word alternately.
+  constexpr int N_READS = 2 * C::TJ + 2 * C::TI;
+  constexpr int READS_PER_ROW = (N_READS + C::TI - 1) / C::TI;
+  // `src` is the byte offset of the stage buffer in smem (wave-uniform, changes every stage): the
+  // per-lane addresses are formed when needed and fragment offsets ride in the instructions' immediates
+  auto read_one = [&](int set, int n, uint32_t src, int step) {
+    const uint8_t* base = smem + src;
+    if (n < 2 * C::TJ) {
+      bf[set][n >> 1][n & 1] = *reinterpret_cast<const int4v*>(base + B_AT + b_off[step][n & 1] + (n >> 1) * 32 * C::B_ROW);
+    } else {
+      const int f = (n - 2 * C::TJ) >> 1;
+      if (((n - 2 * C::TJ) & 1) == 0) af[set][f] = *reinterpret_cast<const int4v*>(base + a_off[step] + f * 32 * C::A_ROW);
+      else if constexpr (ES == 2) idx[set][f] = *reinterpret_cast<const uint16_t*>(base + M_AT + m_off + f * 32 * M_ROW + step * M_STEP);
+      else idx[set][f] = *reinterpret_cast<const int*>(base + M_AT + m_off + f * 32 * M_ROW + step * M_STEP);
     }
   };
-  // stage `st` lives in (sa,sb,sm); the buffer freed by stage st-1 is (na,nb,nm) and receives stage st+2
-  auto pipe_step = [&](int st, uint8_t* sa, uint8_t* sb, uint8_t* sm, uint8_t* na, uint8_t* nb, uint8_t* nm) {
-    // the copies of stage st were issued two stages ago; only those of stage st+1 may still fly
-    if (st + 1 >= nstages) wait_copies_and_barrier<0>();
+  // `half` selects which half of the wave's copies of stage pst is issued between the instructions
+  // (into the buffer at LDS address dst); with `reads`, the fragments of step rstep of the buffer at
+  // offset src go into the other register set.
+  constexpr int PER_SLOT = (NCOPY + 2 * C::TI - 1) / (2 * C::TI);
+  auto mma_step = [&](int set, int half, bool copies, int pst, uint32_t dst, bool reads, uint32_t src, int rstep) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ti = 0; ti < C::TI; ti++) {
+#pragma unroll
+      for (int tj = 0; tj < C::TJ; tj++) {
+        const int4v lo = bf[set][tj][0], hi = bf[set][tj][1];
+        const int8v bfrag = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        acc[ti][tj] = mma32<T>::run(af[set][ti], bfrag, acc[ti][tj], idx[set][ti]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (reads) {
+#pragma unroll
+        for (int u = 0; u < READS_PER_ROW; u++)
+          if (ti * READS_PER_ROW + u < N_READS) read_one(set ^ 1, ti * READS_PER_ROW + u, src, rstep);
+      }
+#pragma unroll
+      for (int u = 0; u < PER_SLOT; u++) {
+        const int q = (half * C::TI + ti) * PER_SLOT + u;
+        if (q < NCOPY && copies) issue_one(q, pst, dst);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  static_assert(C::STEPS == 2, "the pipeline below is written for two instruction steps per stage");
+  auto stage_barrier = [&](bool more) {          // B(st+1): only this wave's copies of stage st+2 may still fly
+    if (!more) wait_copies_and_barrier<0>();
     else if (has_meta_copy) wait_copies_and_barrier<NCOPY>();
     else wait_copies_and_barrier<NCOPY - 1>();
-    compute(sa, sb, sm, st + 2 < nstages, st + 2, na, nb, nm);
   };
 
-  issue(0, s_a0, s_b0, s_m0);
-  if (nstages > 1) issue(1, s_a1, s_b1, s_m1);
-  int st = 0;
-  for (; st + 2 < nstages; st += 3) {
-    pipe_step(st, s_a0, s_b0, s_m0, s_a2, s_b2, s_m2);
-    pipe_step(st + 1, s_a1, s_b1, s_m1, s_a0, s_b0, s_m0);
-    pipe_step(st + 2, s_a2, s_b2, s_m2, s_a1, s_b1, s_m1);
+  issue(0, smem_at);
+  if (nstages > 1) issue(1, smem_at + STAGE_BYTES);
+  stage_barrier(nstages > 1);
+  // stage 0: nothing to multiply yet
+  uint32_t cur = 0, nxt = STAGE_BYTES, fre = 2 * STAGE_BYTES;   // buffers of stage st, st+1, st+2 (= st-1)
+  {
+    const bool more = 2 < nstages;
+#pragma unroll
+    for (int n = 0; n < N_READS; n++) read_one(0, n, cur, 0);
+    if (more) {
+#pragma unroll
+      for (int q = 0; q < C::TI * PER_SLOT && q < NCOPY; q++) issue_one(q, 2, smem_at + fre);
+    }
+    mma_step(0, 1, more, 2, smem_at + fre, true, cur, 1);
+    stage_barrier(more);
   }
-  if (st < nstages) { pipe_step(st, s_a0, s_b0, s_m0, s_a2, s_b2, s_m2); st++; }
-  if (st < nstages) { pipe_step(st, s_a1, s_b1, s_m1, s_a0, s_b0, s_m0); st++; }
+  // stage st: behind B(st), register set 1 holds the last step of stage st-1
+  int st = 1;
+  for (; st + 2 < nstages; st++) {
+    const uint32_t t = cur; cur = nxt; nxt = fre; fre = t;
+    mma_step(1, 0, true, st + 2, smem_at + fre, true, cur, 0);
+    mma_step(0, 1, true, st + 2, smem_at + fre, true, cur, 1);
+    stage_barrier(true);
+  }
+  for (; st < nstages; st++) {                    // the last two stages: nothing left to copy
+    const uint32_t t = cur; cur = nxt; nxt = fre; fre = t;
+    mma_step(1, 0, false, 0, 0, true, cur, 0);
+    mma_step(0, 1, false, 0, 0, true, cur, 1);
+    stage_barrier(false);
+  }
+  mma_step(1, 0, false, 0, 0, false, 0, 0);       // the last step
 
   // ---- split-K: park the float32 accumulators in the workspace, in register order (every group of
   // four accumulators is one contiguous 16-byte-per-lane slab); spmm_reduce_splits finishes the job.
@@ -417,8 +450,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // them out as four full 256-byte row segments per instruction.
   if constexpr (C_JMAJOR && sizeof(OutT) == 2) {
     __syncthreads();                                          // every wave is done with the stage buffers
-    uint8_t* stage = wave < 2 ? s_b0 + wave * 16384 : wave < 4 ? s_b1 + (wave - 2) * 16384
-                   : wave < 6 ? s_b2 + (wave - 4) * 16384 : wave == 6 ? s_a0 : s_a1;
+    uint8_t* stage = smem + wave * 16384;
     const int rr = lane >> 4, chr = lane & 15;
     const int64_t icol = i0 + wi * C::WI + chr * 8;
 #pragma unroll
@@ -456,8 +488,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     // rows.  Stage 128(i) x 64(j) pieces as [i][64 j] (128-byte rows, chunks XOR-swizzled with the
     // row) and stream them out as eight full 128-byte rows per instruction.
     __syncthreads();
-    uint8_t* stage = wave < 2 ? s_b0 + wave * 16384 : wave < 4 ? s_b1 + (wave - 2) * 16384
-                   : wave < 6 ? s_b2 + (wave - 4) * 16384 : wave == 6 ? s_a0 : s_a1;
+    uint8_t* stage = smem + wave * 16384;
     const int rr = lane >> 3, chr = lane & 7;
 #pragma unroll
     for (int half = 0; half < C::TJ / 2; half++) {            // 64 output columns (j) per pass

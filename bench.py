@@ -33,8 +33,26 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
+SETTLE_S = 0.4
+
+
+def settle(fn, seconds=SETTLE_S):
+    """Run fn back to back for `seconds` before a timed region.  The shader clock takes tens of
+    milliseconds of continuous load to leave its idle state and settle at the sustained (power
+    managed) frequency; timings taken in the first ~50 ms of load read 15-20% slow.  Every timed
+    leg (ours, the hipBLASLt comparator, the conversion kernels) is settled the same way."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn(i); i += 1
+        torch.cuda.synchronize()
+
+
 def time_rotating(fn, nsets, iters, warmup):
     """Average device time per call (microseconds) of fn(i % nsets), HIP events on the current stream."""
+    settle(lambda i: fn(i % nsets))
     for i in range(warmup):
         fn(i % nsets)
     start, end = _events(2)
@@ -136,6 +154,7 @@ def spmm_workload(steps, warmup):
     def bwd():
         return torch.mm(dY, w_bwd_t)
 
+    settle(lambda i: (fwd(), bwd()))
     for _ in range(warmup):
         fwd(); bwd()
     ev = [_events(3) for _ in range(steps)]
@@ -151,8 +170,7 @@ def spmm_workload(steps, warmup):
     # dense comparator: hipBLASLt fp16 GEMM on the masked dense weights, same shapes
     Wd_f = w_fwd.to_dense()
     Wd_b = torch.where(tmask, W, torch.zeros_like(W))
-    for _ in range(3):
-        torch.mm(X, Wd_f.t()); torch.mm(dY, Wd_b)
+    settle(lambda i: (torch.mm(X, Wd_f.t()), torch.mm(dY, Wd_b)))
     e = _events(3)
     torch.cuda.synchronize()
     reps = max(3, steps)
@@ -222,6 +240,7 @@ def train_workload(steps, warmup):
                             p.cnt = 0
             opt.step()
             return loss
+        settle(lambda i: step())
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
@@ -269,8 +288,8 @@ def cpu_baseline_spmm(threads):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=["spmm", "train"], default="spmm",
                     help="spmm: BASELINE configs[2] (default, the judged line); train: configs[3] MLP training step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -288,7 +307,7 @@ def main():
         sparse_ms, dense_ms, sl, dl, flops = train_workload(a.steps, a.warmup)
         print(json.dumps({
             "metric": "2:4 sparse MLP training step, dense-equivalent TFLOP/s of its 6 GEMMs", "value": round(flops / (sparse_ms * 1e-3) / 1e12, 2),
-            "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(sparse_ms, 4),
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_s": SETTLE_S, "ms_per_step": round(sparse_ms, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "BASELINE configs[3]: SparseLinearTranspose GPT-2-124M MLP step, 12288 tokens, 768->3072->768, "
                                    "masked decay 2e-4, fused AdamW, mask refresh every 40 steps", "seed": 2},
@@ -302,7 +321,7 @@ def main():
     executed_tflops = (flops / 2) / (dom_ms * 1e-3) / 1e12
     line = {
         "metric": "2:4 spMM TFLOP/s (dense-equivalent 2MNK; fwd X.W^T + transposed dY.W per step)",
-        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_s": SETTLE_S,
         "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "BASELINE configs[2]: fp16 2:4 spMM X[8192,4096].W^T (W[11008,4096]) + dY[8192,11008].W, fp32 accumulate",
