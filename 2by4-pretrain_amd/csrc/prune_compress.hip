@@ -44,15 +44,16 @@ __device__ __forceinline__ float kept_value(uint32_t pos, const float (&x)[4], c
 // panel = false: canonical output, values [m, k/2] and metadata [m, k/8 bytes] row-major; units
 //   (8 dense elements) are walked along rows.
 // panel = true : panel output, [k/KP][m][64 bytes] values and [k/KP][m][KP/8 bytes] metadata with
-//   KP = 128 / sizeof(Out) dense elements per panel.  A block covers 32 rows x 256 dense columns:
-//   32 lanes read 256 consecutive columns of one row (full lines), the two half-waves take adjacent
-//   rows, so that every store instruction writes, per panel, the 2 x 64 contiguous bytes of a row pair.
+//   KP = 128 / sizeof(Out) dense elements per panel.  A block covers 64 rows x 128 dense columns
+//   (32 x 256 when m is not a multiple of 64): 2^lpr_shift lanes read consecutive columns of one row,
+//   the other lanes of the wave take the next rows, so that every store instruction writes, per
+//   panel, the contiguous 64-byte pieces of 4 (2) adjacent rows.
 template <typename In, typename Out, int MODE, typename MaskT>
 __global__ void __launch_bounds__(kThreads)
 prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel) {
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift) {
   constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
   const int64_t upr = k >> 3;                             // 8-element units per row
   const int64_t total = m * upr;
@@ -65,8 +66,9 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     Pack<Out, 4> out;
     int64_t row = 0, col8 = 0, ounit = 0;
     if (panel) {
-      row = (int64_t)blockIdx.x * 32 + it * 8 + (threadIdx.x >> 5);
-      col8 = (int64_t)blockIdx.y * 32 + (threadIdx.x & 31);
+      const int rpi = kThreads >> lpr_shift;                 // rows per iteration
+      row = (int64_t)blockIdx.x * (kUnroll * rpi) + it * rpi + (threadIdx.x >> lpr_shift);
+      col8 = ((int64_t)blockIdx.y << lpr_shift) + (threadIdx.x & ((1 << lpr_shift) - 1));
       live = col8 < upr;                                   // m is a multiple of 32
     }
     if (live) {
@@ -230,10 +232,16 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
     const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == k);
     const int64_t total = m * (k >> 3);
     dim3 grid((unsigned)((total + per_block - 1) / per_block));
-    if (panel) grid = dim3((unsigned)(m / 32), (unsigned)((k + 255) / 256));     // 32 rows x 256 columns per block
+    // lanes per row (log2): 16 lanes read 256 consecutive bytes of bf16 and the four rows of a wave
+    // store 256 contiguous bytes per panel (measured best); 32 lanes when m is not a multiple of 64
+    const int lpr_shift = m % (kUnroll * (kThreads >> 4)) == 0 ? 4 : 5;
+    if (panel) {
+      const int rows_per_block = kUnroll * (kThreads >> lpr_shift), units_per_block = 1 << lpr_shift;
+      grid = dim3((unsigned)(m / rows_per_block), (unsigned)(((k >> 3) + units_per_block - 1) / units_per_block));
+    }
     hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
                        (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta,
-                       contiguous, panel);
+                       contiguous, panel, lpr_shift);
   } else {
     constexpr int R = 16 / sizeof(In);
     dim3 grid((unsigned)((k + 127) / 128), (unsigned)((m + 8 * R - 1) / (8 * R)));

@@ -111,47 +111,55 @@ __device__ __forceinline__ uint32_t search_block(const float (&a)[4][4]) {
 // so the lane reads the block transposed and writes its results transposed.
 template <typename T, bool ABS, bool TRANS>
 __global__ void __launch_bounds__(kThreads)
-transposable_kernel(const T* __restrict__ dense, int64_t ld, int64_t nmajor4, int64_t nminor4,
+transposable_kernel(const T* __restrict__ dense, int64_t ld, int64_t nmajor4, int64_t nminor8,
                     T* __restrict__ sparse, uint8_t* __restrict__ mask_out) {
-  // "major" = the strided dimension in memory, "minor" = the contiguous one
+  // "major" = the strided dimension in memory, "minor" = the contiguous one.  A lane owns two
+  // adjacent 4 x 4 blocks (8 contiguous elements of 4 lines): 16-byte loads and stores for 16-bit
+  // types, 8-byte mask stores.
   const int64_t bminor = (int64_t)blockIdx.y * kThreads + threadIdx.x;
   const int64_t bmajor = blockIdx.x;
-  if (bminor >= nminor4) return;
-  const int64_t off = bmajor * 4 * ld + bminor * 4;
-  Pack<T, 4> in[4];
+  if (bminor >= nminor8) return;
+  const int64_t off = bmajor * 4 * ld + bminor * 8;
+  Pack<T, 8> in[4];
 #pragma unroll
   for (int p = 0; p < 4; p++) in[p].load(dense + off + p * ld);
-  float a[4][4];
+  uint32_t mbits[2];
 #pragma unroll
-  for (int p = 0; p < 4; p++)
+  for (int h = 0; h < 2; h++) {
+    float a[4][4];
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      float v = to_float(in[p].v[e]);
-      if (ABS) v = __builtin_fabsf(v);
-      if (TRANS) a[e][p] = v; else a[p][e] = v;
-    }
-  const uint32_t mbits = search_block(a);
+    for (int p = 0; p < 4; p++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float v = to_float(in[p].v[4 * h + e]);
+        if (ABS) v = __builtin_fabsf(v);
+        if (TRANS) a[e][p] = v; else a[p][e] = v;
+      }
+    mbits[h] = search_block(a);
+  }
 #pragma unroll
   for (int p = 0; p < 4; p++) {
-    uint32_t bytes = 0;
-    Pack<T, 4> out;
+    uint32_t bytes[2] = {0, 0};
+    Pack<T, 8> out;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const int bit = TRANS ? (4 * e + p) : (4 * p + e);
-      const bool keep = (mbits >> bit) & 1;
-      bytes |= (uint32_t)keep << (8 * e);
-      out.v[e] = keep ? in[p].v[e] : T{};
-    }
-    *reinterpret_cast<uint32_t*>(mask_out + off + p * ld) = bytes;
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int bit = TRANS ? (4 * e + p) : (4 * p + e);
+        const bool keep = (mbits[h] >> bit) & 1;
+        bytes[h] |= (uint32_t)keep << (8 * e);
+        out.v[4 * h + e] = keep ? in[p].v[4 * h + e] : T{};
+      }
+    *reinterpret_cast<uint2*>(mask_out + off + p * ld) = make_uint2(bytes[0], bytes[1]);
     if (sparse) out.store(sparse + off + p * ld);
   }
 }
 
 template <typename T, bool ABS, bool TRANS>
 int launch(const void* dense, int64_t ld, int64_t m, int64_t k, void* sparse, uint8_t* mask, hipStream_t s) {
-  const int64_t nmajor4 = (TRANS ? k : m) / 4, nminor4 = (TRANS ? m : k) / 4;
-  dim3 grid((unsigned)nmajor4, (unsigned)((nminor4 + kThreads - 1) / kThreads));
-  hipLaunchKernelGGL((transposable_kernel<T, ABS, TRANS>), grid, dim3(kThreads), 0, s, (const T*)dense, ld, nmajor4, nminor4,
+  const int64_t nmajor4 = (TRANS ? k : m) / 4, nminor8 = (TRANS ? m : k) / 8;     // both extents are multiples of 32
+  dim3 grid((unsigned)nmajor4, (unsigned)((nminor8 + kThreads - 1) / kThreads));
+  hipLaunchKernelGGL((transposable_kernel<T, ABS, TRANS>), grid, dim3(kThreads), 0, s, (const T*)dense, ld, nmajor4, nminor8,
                      (T*)sparse, mask);
   return check_launch("tf24_transposable_mask");
 }
@@ -174,7 +182,7 @@ extern "C" int tf24_transposable_mask_validate(int dtype, int layout, int64_t ld
   if (m <= 0 || m % 32) return fail(TF24_ERR_SHAPE, "%s: number of rows of dense matrix %lld must be divisible by 32", fn, (long long)m);
   if (k <= 0 || k % 64) return fail(TF24_ERR_SHAPE, "%s: number of columns of dense matrix %lld must be divisible by 64", fn, (long long)k);
   const int64_t extent = layout == TF24_ROW_MAJOR ? k : m;
-  if (ld < extent || ld % 4) return fail(TF24_ERR_STRIDE, "%s: leading dimension %lld must be >= %lld and a multiple of 4", fn, (long long)ld, (long long)extent);
+  if (ld < extent || ld % 8) return fail(TF24_ERR_STRIDE, "%s: leading dimension %lld must be >= %lld and a multiple of 8", fn, (long long)ld, (long long)extent);
   if (m > 0x7fffffffLL || k > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "%s: matrix too large", fn);
   return TF24_OK;
 }

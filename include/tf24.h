@@ -112,7 +112,8 @@ int tf24_decompress(const void* values, int dtype, const void* meta, int layout,
  * Transposable 4x4 mask search over the 90 row-and-column 2:4 patterns.
  * Replaces _to_transposable_sparse_semi_structured_kernel and its launcher
  * (sparse/transposable_semi_structured.py:8-47, :50-94) behind TransposableSparse.forward (:198-200).
- *   dense [m,k] dtype (F32|F16|BF16), (layout, ld); m % 32 == 0, k % 64 == 0
+ *   dense [m,k] dtype (F32|F16|BF16), (layout, ld); m % 32 == 0, k % 64 == 0, ld % 8 == 0,
+ *   16-byte aligned base
  *   sparse_out (may be NULL) dense*mask, same dtype/layout/ld;  mask_out bytes (0/1), same layout/ld
  */
 int tf24_transposable_mask(const void* dense, int dtype, int layout, int64_t ld, int64_t m, int64_t k,
