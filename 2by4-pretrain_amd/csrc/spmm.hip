@@ -447,7 +447,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // (8 bytes) in 32 different output rows, so direct stores would touch 32 lines per instruction.
   // Instead every wave stages 64(j) x 128(i) pieces of its sub-tile in a private 16 KB slice of the
   // now idle B stage buffers (256-byte rows, 16-byte chunks XOR-swizzled with the row) and streams
-  // them out as four full 256-byte row segments per instruction.
+  // them out as four full 256-byte row segments per instruction (streaming stores: the tile is not
+  // read again by this kernel and should not displace operand lines in L2).
   if constexpr (C_JMAJOR && sizeof(OutT) == 2) {
     __syncthreads();                                          // every wave is done with the stage buffers
     uint8_t* stage = smem + wave * 16384;
@@ -480,7 +481,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
         const int jl = it * 4 + rr;
         const int64_t jrow = j0 + wj * C::WJ + half * 64 + jl;
         const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 256 + ((chr ^ (jl & 15)) * 16));
-        if (jrow < n_dense && icol < n_sparse) *reinterpret_cast<int4v*>(c + jrow * ldc + icol) = v;
+        if (jrow < n_dense && icol < n_sparse) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + jrow * ldc + icol));
       }
     }
   } else if constexpr (!C_JMAJOR && sizeof(OutT) == 2) {
@@ -516,7 +517,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
         const int il = it * 8 + rr;
         const int64_t irow = i0 + wi * C::WI + il;
         const int4v v = *reinterpret_cast<const int4v*>(stage + il * 128 + ((chr ^ ((il >> 1) & 7)) * 16));
-        if (irow < n_sparse && jcol < n_dense) *reinterpret_cast<int4v*>(c + irow * ldc + jcol) = v;
+        if (irow < n_sparse && jcol < n_dense) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + irow * ldc + jcol));
       }
     }
   } else {
