@@ -217,6 +217,10 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p) {
 __device__ __forceinline__ void g2l16(const uint8_t* g, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
 }
+// same with one dword per lane: lane l writes LDS[base + 4*l]
+__device__ __forceinline__ void g2l4(const uint8_t* g, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
+}
 // s_waitcnt vmcnt(N) + s_barrier with a compile-time N (a bare s_barrier: __syncthreads() would add
 // a fence that drains every outstanding copy)
 template <int N>
@@ -233,8 +237,11 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   constexpr int ES = sizeof(T);
   constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
   constexpr int M_STEP = M_ROW / C::STEPS;
-  constexpr int M_COPIES = C::BI * M_ROW / 1024;            // 1 KB copies per stage: metadata (2 or 4)
-  static_assert(M_COPIES <= C::NW, "one metadata copy per wave at most");
+  // Metadata is copied one dword per lane (256 bytes per wave instruction) so that it can be laid
+  // out step-major in LDS, [step][row][M_STEP bytes]: the index words the 32 rows of a wave read for
+  // one step are then consecutive and conflict-free (row-major, 8 bytes apart, two rows share a bank).
+  constexpr int MW = C::BI * M_ROW / 256 / C::NW;           // dword copies per wave per stage (1 or 2)
+  static_assert(MW * 256 * C::NW == C::BI * M_ROW, "metadata copies must divide among the waves");
   // one stage buffer = [A values | B | A metadata]; three of them rotate
   constexpr int A_STAGE = C::BI * C::A_ROW, B_STAGE = C::BJ * C::B_ROW, M_STAGE = C::BI * M_ROW;
   constexpr int B_AT = A_STAGE, M_AT = A_STAGE + B_STAGE, STAGE_BYTES = A_STAGE + B_STAGE + M_STAGE;
@@ -283,22 +290,24 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     const int ch = (lane & 3) ^ ((row >> 2) & 3);
     ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16 + (int64_t)st_begin * n_sparse * 64;
   }
-  const bool has_meta_copy = wave < M_COPIES;
-  const uint8_t* gm;
-  {
-    const int row = (wave % M_COPIES) * (1024 / M_ROW) + lane * 16 / M_ROW;
-    // a 16-byte copy spans 16/M_ROW rows: clamp so that it never reaches past the last row
-    gm = a_meta + min(i0 + row, n_sparse - 16 / M_ROW) * M_ROW + (lane * 16) % M_ROW + (int64_t)st_begin * n_sparse * M_ROW;
+  const uint8_t* gm[MW];
+#pragma unroll
+  for (int q = 0; q < MW; q++) {
+    const int d = (wave * MW + q) * 64 + lane;               // dword index in the stage's step-major metadata
+    constexpr int DW_PER_STEP = C::BI * M_STEP / 4;
+    const int step = d / DW_PER_STEP, r = d % DW_PER_STEP;
+    const int row = r / (M_STEP / 4), part = r % (M_STEP / 4);
+    gm[q] = a_meta + min(i0 + row, n_sparse - 1) * M_ROW + step * M_STEP + part * 4 + (int64_t)st_begin * n_sparse * M_ROW;
   }
   const int64_t a_stage_stride = n_sparse * 64, m_stage_stride = n_sparse * M_ROW;
-  constexpr int NCOPY = C::NB + C::NA + 1;       // copies per wave per stage (one less without metadata copy)
+  constexpr int NCOPY = C::NB + C::NA + MW;      // copies per wave per stage
 
   // copy q of this wave for stage st into the stage buffer at LDS byte address `dst`
   const uint32_t smem_at = lds_offset(smem);
   auto issue_one = [&](int q, int st, uint32_t dst) {
     if (q < C::NB) g2l16(gb[q] + (int64_t)st * C::B_ROW, dst + B_AT + (wave * C::NB + q) * 1024);
     else if (q < C::NB + C::NA) g2l16(ga[q - C::NB] + (int64_t)st * a_stage_stride, dst + (wave * C::NA + q - C::NB) * 1024);
-    else if (has_meta_copy) g2l16(gm + (int64_t)st * m_stage_stride, dst + M_AT + wave * 1024);
+    else g2l4(gm[q - C::NB - C::NA] + (int64_t)st * m_stage_stride, dst + M_AT + (wave * MW + q - C::NB - C::NA) * 256);
   };
   auto issue = [&](int st, uint32_t dst) {
 #pragma unroll
@@ -323,7 +332,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 #pragma unroll
     for (int h = 0; h < 2; h++) b_off[step][h] = b_row * C::B_ROW + (((step * 4 + h * 2 + lh) ^ b_sw) * 16);
   }
-  const int m_off = a_row * M_ROW + lh * (M_STEP / 2);
+  const int m_off = a_row * M_STEP + lh * (M_STEP / 2);          // inside a step's [row][M_STEP] block
 
   // ---- main loop: a software pipeline over instruction steps.  While the matrix instructions of a
   // step run from one register set, the fragments of the next step are read from LDS into the
@@ -354,8 +363,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     } else {
       const int f = (n - 2 * C::TJ) >> 1;
       if (((n - 2 * C::TJ) & 1) == 0) af[set][f] = *reinterpret_cast<const int4v*>(base + a_off[step] + f * 32 * C::A_ROW);
-      else if constexpr (ES == 2) idx[set][f] = *reinterpret_cast<const uint16_t*>(base + M_AT + m_off + f * 32 * M_ROW + step * M_STEP);
-      else idx[set][f] = *reinterpret_cast<const int*>(base + M_AT + m_off + f * 32 * M_ROW + step * M_STEP);
+      else if constexpr (ES == 2) idx[set][f] = *reinterpret_cast<const uint16_t*>(base + M_AT + m_off + f * 32 * M_STEP + step * (C::BI * M_STEP));
+      else idx[set][f] = *reinterpret_cast<const int*>(base + M_AT + m_off + f * 32 * M_STEP + step * (C::BI * M_STEP));
     }
   };
   // `half` selects which half of the wave's copies of stage pst is issued between the instructions
@@ -389,8 +398,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   static_assert(C::STEPS == 2, "the pipeline below is written for two instruction steps per stage");
   auto stage_barrier = [&](bool more) {          // B(st+1): only this wave's copies of stage st+2 may still fly
     if (!more) wait_copies_and_barrier<0>();
-    else if (has_meta_copy) wait_copies_and_barrier<NCOPY>();
-    else wait_copies_and_barrier<NCOPY - 1>();
+    else wait_copies_and_barrier<NCOPY>();
   };
 
   issue(0, smem_at);
