@@ -15,6 +15,7 @@
 //      range shifted by K/2
 //   D: 16x16: column l%16, rows 4*(l/16)+r;  32x32: column l%32, rows 8*(r/4) + 4*(l/32) + r%4
 #include "tf24_common.hpp"
+#include <type_traits>
 
 namespace tf24 {
 namespace {
@@ -56,6 +57,19 @@ template <> struct mma16<e4m3_t> {
 __device__ __forceinline__ float apply_act(float v, int act) {
   if (act == TF24_ACT_RELU) return v > 0.0f ? v : 0.0f;
   if (act == TF24_ACT_SILU) return v / (1.0f + __expf(-v));
+  return v;
+}
+
+// The output pass of the tiled kernel is compiled three times: without bias and activation, with a
+// bias only, and with both decided at run time.  Left to run-time tests alone, the per-element
+// selects and the inlined SiLU more than triple the time of the pass (21 000 against 6 300 cycles
+// per 256 x 256 tile), which is a tenth of the whole kernel at k = 4096.
+enum { EPI_PLAIN = 0, EPI_BIAS = 1, EPI_RUNTIME = 2 };
+template <int MODE, typename OutT>
+__device__ __forceinline__ float finish_element(float accv, float scale, const OutT* bias, int64_t row, bool row_ok, int act) {
+  float v = accv * scale;
+  if constexpr (MODE == EPI_BIAS) { if (row_ok) v += to_float(bias[row]); }
+  if constexpr (MODE == EPI_RUNTIME) { if (bias && row_ok) v += to_float(bias[row]); v = apply_act(v, act); }
   return v;
 }
 
@@ -450,110 +464,110 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     return;
   }
 
-  // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
-  // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
-  // (8 bytes) in 32 different output rows, so direct stores would touch 32 lines per instruction.
-  // Instead every wave stages 64(j) x 128(i) pieces of its sub-tile in a private 16 KB slice of the
-  // now idle B stage buffers (256-byte rows, 16-byte chunks XOR-swizzled with the row) and streams
-  // them out as four full 256-byte row segments per instruction (streaming stores: the tile is not
-  // read again by this kernel and should not displace operand lines in L2).
-  if constexpr (C_JMAJOR && sizeof(OutT) == 2) {
-    __syncthreads();                                          // every wave is done with the stage buffers
-    uint8_t* stage = smem + wave * 16384;
-    const int rr = lane >> 4, chr = lane & 15;
-    const int64_t icol = i0 + wi * C::WI + chr * 8;
-#pragma unroll
-    for (int half = 0; half < C::TJ / 2; half++) {            // 64 output rows (j) per pass
-#pragma unroll
+  auto output_pass = [&](auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
+    // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
+    // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
+    // (8 bytes) in 32 different output rows, so direct stores would touch 32 lines per instruction.
+    // Instead every wave stages 64(j) x 128(i) pieces of its sub-tile in a private 16 KB slice of the
+    // now idle B stage buffers (256-byte rows, 16-byte chunks XOR-swizzled with the row) and streams
+    // them out as four full 256-byte row segments per instruction (streaming stores: the tile is not
+    // read again by this kernel and should not displace operand lines in L2).
+    if constexpr (C_JMAJOR && sizeof(OutT) == 2) {
+      __syncthreads();                                          // every wave is done with the stage buffers
+      uint8_t* stage = smem + wave * 16384;
+      const int rr = lane >> 4, chr = lane & 15;
+      const int64_t icol = i0 + wi * C::WI + chr * 8;
+  #pragma unroll
+      for (int half = 0; half < C::TJ / 2; half++) {            // 64 output rows (j) per pass
+  #pragma unroll
+        for (int ti = 0; ti < C::TI; ti++)
+  #pragma unroll
+          for (int t2 = 0; t2 < 2; t2++) {
+            const int tj = half * 2 + t2;
+            const int jl = t2 * 32 + l32;
+  #pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+              OutT o[4];
+  #pragma unroll
+              for (int r = 0; r < 4; r++) {
+                o[r] = from_float<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
+              }
+              const int ch = ti * 4 + g;
+              *reinterpret_cast<Pack<OutT, 4>*>(stage + jl * 256 + ((ch ^ (jl & 15)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+            }
+          }
+  #pragma unroll
+        for (int it = 0; it < 16; it++) {
+          const int jl = it * 4 + rr;
+          const int64_t jrow = j0 + wj * C::WJ + half * 64 + jl;
+          const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 256 + ((chr ^ (jl & 15)) * 16));
+          if (jrow < n_dense && icol < n_sparse) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + jrow * ldc + icol));
+        }
+      }
+    } else if constexpr (!C_JMAJOR && sizeof(OutT) == 2) {
+      // i-major 16-bit output (the W.B of `S @ dense`): a lane owns single elements of 64+ different
+      // rows.  Stage 128(i) x 64(j) pieces as [i][64 j] (128-byte rows, chunks XOR-swizzled with the
+      // row) and stream them out as eight full 128-byte rows per instruction.
+      __syncthreads();
+      uint8_t* stage = smem + wave * 16384;
+      const int rr = lane >> 3, chr = lane & 7;
+  #pragma unroll
+      for (int half = 0; half < C::TJ / 2; half++) {            // 64 output columns (j) per pass
+  #pragma unroll
+        for (int ti = 0; ti < C::TI; ti++)
+  #pragma unroll
+          for (int t2 = 0; t2 < 2; t2++) {
+            const int tj = half * 2 + t2;
+            const int jl = t2 * 32 + l32;
+  #pragma unroll
+            for (int g = 0; g < 4; g++)
+  #pragma unroll
+              for (int r = 0; r < 4; r++) {
+                const int il = ti * 32 + g * 8 + lh * 4 + r;
+                const int64_t row = i0 + wi * C::WI + il;
+                *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ ((il >> 1) & 7)) * 16) + (jl & 7) * 2) =
+                    from_float<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row, row < n_sparse, act));
+              }
+          }
+        const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
+  #pragma unroll
+        for (int it = 0; it < 16; it++) {
+          const int il = it * 8 + rr;
+          const int64_t irow = i0 + wi * C::WI + il;
+          const int4v v = *reinterpret_cast<const int4v*>(stage + il * 128 + ((chr ^ ((il >> 1) & 7)) * 16));
+          if (irow < n_sparse && jcol < n_dense) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + irow * ldc + jcol));
+        }
+      }
+    } else {
+  #pragma unroll
       for (int ti = 0; ti < C::TI; ti++)
-#pragma unroll
-        for (int t2 = 0; t2 < 2; t2++) {
-          const int tj = half * 2 + t2;
-          const int jl = t2 * 32 + l32;
-#pragma unroll
+  #pragma unroll
+        for (int tj = 0; tj < C::TJ; tj++) {
+          const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
+  #pragma unroll
           for (int g = 0; g < 4; g++) {
             const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+            if (col >= n_dense || row >= n_sparse) continue;
             OutT o[4];
-#pragma unroll
+  #pragma unroll
             for (int r = 0; r < 4; r++) {
-              float v = acc[ti][tj][g * 4 + r] * scale;
-              if (bias && row < n_sparse) v += to_float(bias[row + r]);
-              o[r] = from_float<OutT>(apply_act(v, act));
+              o[r] = from_float<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, true, act));
             }
-            const int ch = ti * 4 + g;
-            *reinterpret_cast<Pack<OutT, 4>*>(stage + jl * 256 + ((ch ^ (jl & 15)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
-          }
-        }
-#pragma unroll
-      for (int it = 0; it < 16; it++) {
-        const int jl = it * 4 + rr;
-        const int64_t jrow = j0 + wj * C::WJ + half * 64 + jl;
-        const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 256 + ((chr ^ (jl & 15)) * 16));
-        if (jrow < n_dense && icol < n_sparse) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + jrow * ldc + icol));
-      }
-    }
-  } else if constexpr (!C_JMAJOR && sizeof(OutT) == 2) {
-    // i-major 16-bit output (the W.B of `S @ dense`): a lane owns single elements of 64+ different
-    // rows.  Stage 128(i) x 64(j) pieces as [i][64 j] (128-byte rows, chunks XOR-swizzled with the
-    // row) and stream them out as eight full 128-byte rows per instruction.
-    __syncthreads();
-    uint8_t* stage = smem + wave * 16384;
-    const int rr = lane >> 3, chr = lane & 7;
-#pragma unroll
-    for (int half = 0; half < C::TJ / 2; half++) {            // 64 output columns (j) per pass
-#pragma unroll
-      for (int ti = 0; ti < C::TI; ti++)
-#pragma unroll
-        for (int t2 = 0; t2 < 2; t2++) {
-          const int tj = half * 2 + t2;
-          const int jl = t2 * 32 + l32;
-#pragma unroll
-          for (int g = 0; g < 4; g++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-              const int il = ti * 32 + g * 8 + lh * 4 + r;
-              const int64_t row = i0 + wi * C::WI + il;
-              float v = acc[ti][tj][g * 4 + r] * scale;
-              if (bias && row < n_sparse) v += to_float(bias[row]);
-              *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ ((il >> 1) & 7)) * 16) + (jl & 7) * 2) =
-                  from_float<OutT>(apply_act(v, act));
+            if constexpr (C_JMAJOR) {
+              *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+            } else {
+  #pragma unroll
+              for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
             }
+          }
         }
-      const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
-#pragma unroll
-      for (int it = 0; it < 16; it++) {
-        const int il = it * 8 + rr;
-        const int64_t irow = i0 + wi * C::WI + il;
-        const int4v v = *reinterpret_cast<const int4v*>(stage + il * 128 + ((chr ^ ((il >> 1) & 7)) * 16));
-        if (irow < n_sparse && jcol < n_dense) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + irow * ldc + jcol));
-      }
     }
-  } else {
-#pragma unroll
-    for (int ti = 0; ti < C::TI; ti++)
-#pragma unroll
-      for (int tj = 0; tj < C::TJ; tj++) {
-        const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
-          if (col >= n_dense || row >= n_sparse) continue;
-          OutT o[4];
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            float v = acc[ti][tj][g * 4 + r] * scale;
-            if (bias) v += to_float(bias[row + r]);
-            o[r] = from_float<OutT>(apply_act(v, act));
-          }
-          if constexpr (C_JMAJOR) {
-            *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
-          } else {
-#pragma unroll
-            for (int r = 0; r < 4; r++) c[(row + r) * ldc + col] = o[r];
-          }
-        }
-      }
-  }
+  };
+  if (!bias && act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_PLAIN>{});
+  else if (act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_BIAS>{});
+  else output_pass(std::integral_constant<int, EPI_RUNTIME>{});
 }
 
 // Second pass of a split-K product: a block handles one eighth of a tile (the accumulator groups
