@@ -162,3 +162,60 @@ def test_functional_linear_entry_point(cuda):
     assert torch.allclose(out.float().cpu(), ref_silu, rtol=2e-3, atol=2e-3)
     with pytest.raises(RuntimeError):
         sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="gelu")
+
+
+def test_my_linear_and_sparse_linear_modules(cuda):
+    """sparse/sparse_ops.py: MyLinear is nn.Linear; SparseLinear has the same forward and weight/bias
+    gradients, and dX = dY . MVUE24(W^T)^T with the uniforms of torch's generator."""
+    import sparse
+    torch.manual_seed(3)
+    ref = torch.nn.Linear(128, 64).to(cuda)
+    x = torch.randn(8, 16, 128, device=cuda)
+    gy = torch.randn(8, 16, 64, device=cuda)
+    for cls in (sparse.MyLinear, sparse.SparseLinear):
+        mod = cls(128, 64).to(cuda)
+        mod.load_state_dict(ref.state_dict())
+        xr, xm = x.clone().requires_grad_(), x.clone().requires_grad_()
+        yr, ym = ref(xr), mod(xm)
+        assert torch.allclose(ym, yr, atol=1e-5, rtol=1e-5)
+        ref.zero_grad()
+        yr.backward(gy)
+        torch.manual_seed(11)
+        ym.backward(gy)
+        assert torch.allclose(mod.weight.grad, ref.weight.grad, atol=1e-4, rtol=1e-4)
+        assert torch.allclose(mod.bias.grad, ref.bias.grad, atol=1e-4, rtol=1e-4)
+        if cls is sparse.MyLinear:
+            assert torch.allclose(xm.grad, xr.grad, atol=1e-5, rtol=1e-5)
+        else:
+            torch.manual_seed(11)
+            w_est = sparse.MVUE24_approx_triton(mod.weight.detach().t()).t()
+            want = (gy.reshape(-1, 64) @ w_est).view_as(x)
+            assert torch.allclose(xm.grad, want, atol=1e-5, rtol=1e-5)
+            assert ((w_est != 0).t().reshape(-1, 4).sum(-1) <= 2).all()        # 2:4 along the output axis
+
+
+def test_soft_threshold_linear_module(cuda):
+    """README S-STE recipe: forward uses scale * soft_threshold24(W); the gradient passes straight
+    through to W; init_scale is the least-squares scale."""
+    import sparse
+    torch.manual_seed(4)
+    mod = sparse.SoftThresholdLinear(128, 64).to(cuda)
+    mod.init_scale()
+    w = mod.weight.detach()
+    ws, _ = oracle.soft_threshold24(w.cpu())
+    want_scale = (w.cpu().flatten() @ ws.flatten()) / (ws.flatten() @ ws.flatten())
+    assert abs(mod.scale.item() - want_scale.item()) < 1e-5 and mod.scale.item() > 1.0
+    x = torch.randn(32, 128, device=cuda)
+    y = mod(x)
+    want = F.linear(x, ws.to(cuda) * mod.scale, mod.bias)
+    assert torch.allclose(y, want, atol=1e-5, rtol=1e-5)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    assert torch.allclose(mod.weight.grad, gy.t() @ x, atol=1e-4, rtol=1e-4)     # straight-through
+    # STEP recipe: magnitude-pruned weight with a straight-through gradient
+    w2 = torch.randn(64, 128, device=cuda, requires_grad=True)
+    sp = sparse.Sparse24.apply(w2)
+    want_sp, _ = oracle.sparse24_dense(w2.detach().cpu())
+    assert sp.detach().cpu().equal(want_sp)
+    sp.backward(torch.ones_like(sp))
+    assert w2.grad.equal(torch.ones_like(w2))
