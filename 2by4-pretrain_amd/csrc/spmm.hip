@@ -57,6 +57,7 @@ template <> struct mma16<e4m3_t> {
 __device__ __forceinline__ float apply_act(float v, int act) {
   if (act == TF24_ACT_RELU) return v > 0.0f ? v : 0.0f;
   if (act == TF24_ACT_SILU) return v / (1.0f + __expf(-v));
+  if (act == TF24_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
   return v;
 }
 
@@ -713,7 +714,7 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
   if (ldb < bext || ldb % dmult) return fail(TF24_ERR_STRIDE, "%s: ldb %lld must be >= %lld and a multiple of %lld", fn, (long long)ldb, (long long)bext, (long long)dmult);
   const int64_t cext = c_layout == TF24_ROW_MAJOR ? n_dense : n_sparse;
   if (ldc < cext || ldc % 4) return fail(TF24_ERR_STRIDE, "%s: ldc %lld must be >= %lld and a multiple of 4", fn, (long long)ldc, (long long)cext);
-  if (activation < TF24_ACT_NONE || activation > TF24_ACT_SILU) return fail(TF24_ERR_ARG, "%s: bad activation %d", fn, activation);
+  if (activation < TF24_ACT_NONE || activation > TF24_ACT_GELU) return fail(TF24_ERR_ARG, "%s: bad activation %d", fn, activation);
   return TF24_OK;
 }
 

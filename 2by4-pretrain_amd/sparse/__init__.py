@@ -7,6 +7,7 @@ is missing -- there is no CPU or PyTorch fallback.
 from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured
 from .transposable_semi_structured import TransposableSparse, mask_select
 from .decay import masked_add_
+from .adamw import MaskedDecayAdamW
 from .dense_ops import (soft_threshold24, sparse24, MVUE24_approx,
                         soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton)
 from .sparse_linear_transpose import SparseLinearTranspose, sparse_linear_transpose
@@ -16,7 +17,7 @@ from .sparse_ops import MyLinear, SparseLinear, SoftThreshold, SoftThresholdLine
 __all__ = [
     "SparseSemiStructuredTensor", "to_sparse_semi_structured",
     "TransposableSparse", "mask_select",
-    "masked_add_",
+    "masked_add_", "MaskedDecayAdamW",
     "soft_threshold24", "sparse24", "MVUE24_approx",
     "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
     "SparseLinearTranspose", "sparse_linear_transpose",

@@ -15,7 +15,7 @@ _lib = None
 F32, F16, BF16, E4M3, U8 = 0, 1, 2, 3, 4
 ROW_MAJOR, COL_MAJOR = 0, 1
 PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE = 0, 1, 2
-ACT_NONE, ACT_RELU, ACT_SILU = 0, 1, 2
+ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
 COMPRESSED_CANONICAL, COMPRESSED_PANEL = 0, 1
 
 _DTYPES = {
@@ -27,6 +27,7 @@ _i = ctypes.c_int
 _i64 = ctypes.c_int64
 _p = ctypes.c_void_p
 _f = ctypes.c_float
+_d = ctypes.c_double
 
 _SIGNATURES = {
     "tf24_version": (ctypes.c_char_p, []),
@@ -40,6 +41,7 @@ _SIGNATURES = {
     "tf24_sparse24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _p, _p]),
     "tf24_mvue24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _i64, _p, _p]),
     "tf24_masked_add": (_i, [_p, _i, _p, _i, _p, _i, _i64, _f, _p]),
+    "tf24_adamw_masked_decay": (_i, [_p, _p, _i, _p, _p, _p, _i, _i64, _d, _d, _d, _d, _d, _d, _i64, _p]),
     "tf24_spmm": (_i, [_p, _p, _i, _i, _i64, _i64, _p, _i, _i64, _i64, _p, _i, _i, _i64, _p, _f, _i, _p, _i64, _p]),
     "tf24_spmm_workspace_bytes": (_i64, [_i, _i64, _i64, _i64]),
     "tf24_transpose": (_i, [_p, _i, _i64, _i64, _i64, _p, _i64, _p]),

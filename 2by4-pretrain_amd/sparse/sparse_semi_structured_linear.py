@@ -18,14 +18,14 @@ from .semi_structured import SparseSemiStructuredTensor, _spmm
 
 __all__ = ["sparse_semi_structured_linear"]
 
-_ACTIVATIONS = {None: N.ACT_NONE, "none": N.ACT_NONE, "relu": N.ACT_RELU, "silu": N.ACT_SILU}
+_ACTIVATIONS = {None: N.ACT_NONE, "none": N.ACT_NONE, "relu": N.ACT_RELU, "silu": N.ACT_SILU, "gelu": N.ACT_GELU}
 
 
 def sparse_semi_structured_linear(input: torch.Tensor, weight, meta: Optional[torch.Tensor] = None,
                                   bias: Optional[torch.Tensor] = None, activation: Optional[str] = None,
                                   out_dtype: Optional[torch.dtype] = None, scale: float = 1.0) -> torch.Tensor:
     if activation not in _ACTIVATIONS:
-        raise RuntimeError(f"activation {activation!r} is not supported (none, relu, silu)")
+        raise RuntimeError(f"activation {activation!r} is not supported (none, relu, silu, gelu)")
     if not isinstance(weight, SparseSemiStructuredTensor):
         if meta is None:
             raise RuntimeError("sparse_semi_structured_linear: metadata tensor missing")

@@ -53,7 +53,8 @@ typedef enum {
   TF24_PRUNE_MVUE = 2       /* MVUE24 sampling from a supplied U(0,1) tensor */
 } tf24_prune_mode;
 
-typedef enum { TF24_ACT_NONE = 0, TF24_ACT_RELU = 1, TF24_ACT_SILU = 2 } tf24_activation;
+/* GELU is the exact (erf) form, torch.nn.functional.gelu's default; the reference's epilogues stop at SILU */
+typedef enum { TF24_ACT_NONE = 0, TF24_ACT_RELU = 1, TF24_ACT_SILU = 2, TF24_ACT_GELU = 3 } tf24_activation;
 
 /*
  * Storage of a compressed [m,k] matrix (values + metadata).
@@ -135,6 +136,18 @@ int tf24_sparse24_dense(const void* dense, int dtype, int layout, int64_t ld, in
                         void* sparse_out, void* mask_out, void* stream);
 int tf24_mvue24_dense(const void* dense, int dtype, int layout, int64_t ld, int64_t m, int64_t k,
                       const float* rand, int64_t rand_ld, void* sparse_out, void* stream);
+
+/*
+ * AdamW step with the masked decay folded in: one pass instead of masked_add_ followed by the
+ * optimizer.  Follows the reference's optimizer (sparse/adamw.py:70-113: decoupled weight decay,
+ * bias-corrected moments, no amsgrad) with the decay of sparse/decay.py:27-37 applied to the
+ * gradient first, as the training loop of README.md:205-213 does; the gradient is only read.
+ *   p, exp_avg, exp_avg_sq F32 in place; grad F32|F16|BF16; mask U8|F32|F16|BF16 or NULL (no decay)
+ *   step = number of this update, starting at 1
+ */
+int tf24_adamw_masked_decay(float* p, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
+                            const void* mask, int mask_dtype, int64_t n, double lr, double beta1, double beta2,
+                            double eps, double weight_decay, double decay_alpha, int64_t step, void* stream);
 
 /*
  * Masked decay, in place: grad[i] += alpha * p[i] where mask[i] == 0.

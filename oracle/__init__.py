@@ -27,4 +27,5 @@ from .transposable import (  # noqa: F401
     transposable_patterns, transposable_mask, transposable_mask_bruteforce,
 )
 from .decay import masked_add  # noqa: F401
+from .adamw import adamw_masked_decay  # noqa: F401
 from .spmm import spmm_ref, linear_ref  # noqa: F401

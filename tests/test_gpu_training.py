@@ -160,8 +160,10 @@ def test_functional_linear_entry_point(cuda):
     out = sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="silu")
     ref_silu = F.silu(oracle.linear_ref(x, wm))
     assert torch.allclose(out.float().cpu(), ref_silu, rtol=2e-3, atol=2e-3)
+    out = sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="gelu")          # exact (erf) GELU
+    assert torch.allclose(out.float().cpu(), F.gelu(oracle.linear_ref(x, wm)), rtol=2e-3, atol=2e-3)
     with pytest.raises(RuntimeError):
-        sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="gelu")
+        sparse.sparse_semi_structured_linear(x.to(cuda), s, activation="tanh")
 
 
 def test_my_linear_and_sparse_linear_modules(cuda):
@@ -219,3 +221,44 @@ def test_soft_threshold_linear_module(cuda):
     assert sp.detach().cpu().equal(want_sp)
     sp.backward(torch.ones_like(sp))
     assert w2.grad.equal(torch.ones_like(w2))
+
+
+@pytest.mark.parametrize("gdt", [torch.float32, torch.float16])
+def test_masked_decay_adamw_kernel(cuda, gdt):
+    """One fused pass against the oracle (float32; rtol 2e-6: torch's CPU ops may contract a
+    multiply-add that the kernel rounds twice) and against the two-pass recipe it replaces."""
+    import sparse
+    g = torch.Generator().manual_seed(31)
+    hyp = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    p0 = torch.randn(96, 200, generator=g)                      # 19200 elements + odd tail coverage below
+    mask = torch.rand(96, 200, generator=g) > 0.5
+    par = torch.nn.Parameter(p0.clone().to(cuda))
+    par.mask, par.mode, par.cnt = mask.to(cuda), "sparse", 3
+    plain = torch.nn.Parameter(torch.randn(1003, generator=g).to(cuda))        # no mask, unaligned tail
+    if gdt != torch.float32:
+        par.grad_dtype = plain.grad_dtype = None                 # let the float32 parameters hold half gradients
+    opt = sparse.MaskedDecayAdamW([par, plain], alpha=2e-4, **hyp)
+    ref_par = torch.nn.Parameter(p0.clone().to(cuda))
+    ref_plain = torch.nn.Parameter(plain.detach().clone())
+    ref_opt = torch.optim.AdamW([ref_par, ref_plain], foreach=False, fused=False, **hyp)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    q, qm, qv = plain.detach().cpu().clone(), torch.zeros(1003), torch.zeros(1003)
+    for step in range(1, 5):
+        grad = torch.randn(96, 200, generator=g).to(gdt)
+        grad2 = torch.randn(1003, generator=g).to(gdt)
+        par.grad, plain.grad = grad.to(cuda), grad2.to(cuda)
+        opt.step()
+        assert par.cnt == 0
+        p, m, v = oracle.adamw_masked_decay(p, grad, m, v, mask, step, alpha=2e-4, **hyp)
+        q, qm, qv = oracle.adamw_masked_decay(q, grad2, qm, qv, None, step, **hyp)
+        assert torch.allclose(par.detach().cpu(), p, rtol=2e-6, atol=1e-8)
+        assert torch.allclose(opt.state[par]["exp_avg"].cpu(), m, rtol=2e-6, atol=1e-10)
+        assert torch.allclose(opt.state[par]["exp_avg_sq"].cpu(), v, rtol=2e-6, atol=1e-12)
+        assert torch.allclose(plain.detach().cpu(), q, rtol=2e-6, atol=1e-8)
+        # the recipe it replaces: masked_add_ on the float32 gradient, then an AdamW step
+        ref_par.grad = grad.to(cuda).float()
+        sparse.masked_add_(ref_par.grad, ref_par.data, par.mask, alpha=2e-4)
+        ref_plain.grad = grad2.to(cuda).float()
+        ref_opt.step()
+        assert torch.allclose(par.detach(), ref_par.detach(), rtol=1e-5, atol=1e-7)
+        assert torch.allclose(plain.detach(), ref_plain.detach(), rtol=1e-5, atol=1e-7)

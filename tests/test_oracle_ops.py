@@ -191,3 +191,32 @@ def test_masked_add_docstring_equivalence():
     out = oracle.masked_add(grad, p, mask, alpha=2e-4)
     assert torch.allclose(out, want, rtol=0, atol=1e-9)
     assert out[mask].equal(grad[mask])
+
+
+# ------------------------------------------------------------------ AdamW with masked decay
+def test_adamw_oracle_matches_torch_adamw_and_closed_form():
+    """The oracle's AdamW against torch.optim.AdamW (an independent implementation of the same
+    update) over several steps, and the first step's closed form."""
+    g = torch.Generator().manual_seed(21)
+    p0 = torch.randn(64, 96, generator=g)
+    hyp = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    ref_p = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([ref_p], foreach=False, fused=False, **hyp)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    for step in range(1, 6):
+        grad = torch.randn(64, 96, generator=g)
+        ref_p.grad = grad.clone()
+        opt.step()
+        p_prev = p
+        p, m, v = oracle.adamw_masked_decay(p, grad, m, v, None, step, **hyp)
+        assert torch.allclose(p, ref_p.detach(), rtol=1e-5, atol=1e-7)
+        if step == 1:       # m = (1-b1) g, v = (1-b2) g^2: update = -lr * g / (|g| + eps * sqrt(1-b2)... ) ~ -lr * sign(g)
+            want = p_prev * (1 - hyp["lr"] * hyp["weight_decay"]) - hyp["lr"] * grad / (grad.abs() + hyp["eps"])
+            assert torch.allclose(p, want, rtol=1e-5, atol=1e-7)
+    # the decay term enters through the gradient exactly as masked_add_ followed by the plain update
+    mask = torch.rand(64, 96, generator=g) > 0.5
+    grad = torch.randn(64, 96, generator=g)
+    a = oracle.adamw_masked_decay(p, grad, m, v, mask, 6, alpha=2e-4, **hyp)
+    b = oracle.adamw_masked_decay(p, oracle.masked_add(grad, p, mask, 2e-4), m, v, None, 6, **hyp)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
