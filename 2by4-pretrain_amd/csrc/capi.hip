@@ -55,10 +55,10 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
                                             int out_dtype) {
   const char* fn = "tf24_prune_compress";
   if (!is_float_dtype(in_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
-  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && out_dtype != TF24_E4M3)
+  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && !is_float8(out_dtype))
     return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
   if (!is_layout(layout)) return fail(TF24_ERR_ARG, "%s: bad layout %d", fn, layout);
-  const int64_t min_rows = 32, min_cols = out_dtype == TF24_E4M3 ? 128 : 64;
+  const int64_t min_rows = 32, min_cols = is_float8(out_dtype) ? 128 : 64;
   if (m < min_rows || m % min_rows || k < min_cols || k % min_cols)
     return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld) is not supported: both dimensions must be >= and a multiple of (%lld, %lld)",
                 fn, (long long)m, (long long)k, (long long)min_rows, (long long)min_cols);

@@ -52,17 +52,18 @@ int launch(const void* values, const void* meta, bool panel, int64_t m, int64_t 
 extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, int layout, int64_t m, int64_t k,
                                void* dense_out, void* stream) {
   using namespace tf24;
-  const int64_t mult = dtype == TF24_E4M3 ? 32 : 16;
+  const int64_t mult = is_float8(dtype) ? 32 : 16;
   if (m <= 0 || k <= 0 || k % mult) return fail(TF24_ERR_SHAPE, "tf24_decompress: k=%lld must be a positive multiple of %lld", (long long)k, (long long)mult);
   if (!values || !meta || !dense_out) return fail(TF24_ERR_ARG, "tf24_decompress: null pointer");
   if (layout != TF24_COMPRESSED_CANONICAL && layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_decompress: bad compressed layout %d", layout);
   const bool panel = layout == TF24_COMPRESSED_PANEL;
-  if (panel && k % (dtype == TF24_E4M3 ? 128 : 64)) return fail(TF24_ERR_SHAPE, "tf24_decompress: panel layout needs whole panels (k=%lld)", (long long)k);
+  if (panel && k % (is_float8(dtype) ? 128 : 64)) return fail(TF24_ERR_SHAPE, "tf24_decompress: panel layout needs whole panels (k=%lld)", (long long)k);
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case TF24_F16: return launch<f16_t>(values, meta, panel, m, k, dense_out, s);
     case TF24_BF16: return launch<bf16_t>(values, meta, panel, m, k, dense_out, s);
     case TF24_E4M3: return launch<e4m3_t>(values, meta, panel, m, k, dense_out, s);
+    case TF24_E5M2: return launch<e5m2_t>(values, meta, panel, m, k, dense_out, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_decompress: unsupported dtype %d", dtype);
 }

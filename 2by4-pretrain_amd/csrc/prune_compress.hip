@@ -288,6 +288,7 @@ int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t
     case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
     case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
     case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported output dtype %d", out_dtype);
 }

@@ -53,6 +53,13 @@ template <> struct mma16<e4m3_t> {
     return __builtin_amdgcn_smfmac_f32_16x16x128_fp8_fp8(a, b, c, idx, 0, 0);
   }
 };
+template <> struct mma16<e5m2_t> {
+  static constexpr int KSTEP = 128;
+  template <int ABID>
+  static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
+    return __builtin_amdgcn_smfmac_f32_16x16x128_bf8_bf8(a, b, c, idx, 0, 0);
+  }
+};
 
 __device__ __forceinline__ float apply_act(float v, int act) {
   if (act == TF24_ACT_RELU) return v > 0.0f ? v : 0.0f;
@@ -198,6 +205,11 @@ template <> struct mma32<bf16_t> {
 template <> struct mma32<e4m3_t> {
   static __device__ __forceinline__ float16v run(int4v a, int8v b, float16v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(a, b, c, idx, 0, 0);
+  }
+};
+template <> struct mma32<e5m2_t> {
+  static __device__ __forceinline__ float16v run(int4v a, int8v b, float16v c, int idx) {
+    return __builtin_amdgcn_smfmac_f32_32x32x64_bf8_bf8(a, b, c, idx, 0, 0);
   }
 };
 
@@ -701,9 +713,9 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
                                   int out_dtype, int c_layout, int64_t ldc, int activation) {
   using namespace tf24;
   const char* fn = "tf24_spmm";
-  if (dtype != TF24_F16 && dtype != TF24_BF16 && dtype != TF24_E4M3) return fail(TF24_ERR_DTYPE, "%s: unsupported operand dtype %d", fn, dtype);
+  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_float8(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported operand dtype %d", fn, dtype);
   if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && out_dtype != TF24_F32) return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
-  const bool eight = dtype == TF24_E4M3;
+  const bool eight = is_float8(dtype);
   const int64_t kmult = eight ? 128 : 64, dmult = eight ? 16 : 8;
   if (n_sparse <= 0 || n_sparse % 32) return fail(TF24_ERR_SHAPE, "%s: sparse operand rows %lld must be a positive multiple of 32", fn, (long long)n_sparse);
   if (k <= 0 || k % kmult) return fail(TF24_ERR_SHAPE, "%s: inner dimension %lld must be a positive multiple of %lld", fn, (long long)k, (long long)kmult);
@@ -722,7 +734,7 @@ extern "C" int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_
   using namespace tf24;
   const int64_t big = (int64_t)1 << 40;
   int splits;
-  if (dtype == TF24_E4M3) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
+  if (is_float8(dtype)) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
   else splits = choose_splits<f16_t, TiledCfg>(n_sparse, k, n_dense, big);
   if (splits < 2) return 0;
   const int64_t tiles = ((n_sparse + TiledCfg::BI - 1) / TiledCfg::BI) * ((n_dense + TiledCfg::BJ - 1) / TiledCfg::BJ);
@@ -743,6 +755,7 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout,
   switch (dtype) {
     case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
     case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    case TF24_E5M2: return dispatch_out<e5m2_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
     default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
   }
 }

@@ -16,12 +16,15 @@ int check_launch(const char* what);
 struct f16_t { uint16_t bits; };
 struct bf16_t { uint16_t bits; };
 struct e4m3_t { uint8_t bits; };
+struct e5m2_t { uint8_t bits; };
 
 template <typename T> struct dtype_of;
 template <> struct dtype_of<float> { static constexpr int value = TF24_F32; };
 template <> struct dtype_of<f16_t> { static constexpr int value = TF24_F16; };
 template <> struct dtype_of<bf16_t> { static constexpr int value = TF24_BF16; };
 template <> struct dtype_of<e4m3_t> { static constexpr int value = TF24_E4M3; };
+template <> struct dtype_of<e5m2_t> { static constexpr int value = TF24_E5M2; };
+__host__ __device__ inline bool is_float8(int dt) { return dt == TF24_E4M3 || dt == TF24_E5M2; }
 template <> struct dtype_of<uint8_t> { static constexpr int value = TF24_U8; };
 
 __host__ __device__ inline int dtype_size(int dt) {
@@ -82,6 +85,31 @@ __host__ __device__ inline float e4m3_to_float(uint8_t b) {
   return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) | sign);
 }
 __device__ __forceinline__ float to_float(e4m3_t v) { return e4m3_to_float(v.bits); }
+
+// OCP e5m2 (bias 15, infinities, NaN): the upper byte of an IEEE half.  Round to nearest even from
+// float32 on the bit pattern: magnitudes of 2^16 and above become infinity (the rounding carries
+// 61440..65535 there as well), subnormals (below 2^-14) are rounded by a float32 addition.
+__host__ __device__ inline uint8_t float_to_e5m2(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  u &= 0x7fffffffu;
+  uint32_t r;
+  if (u >= (143u << 23)) {
+    r = u > 0x7f800000u ? 0x7fu : 0x7cu;
+  } else if (u < (113u << 23)) {
+    const float v = __builtin_bit_cast(float, u) + __builtin_bit_cast(float, 134u << 23);
+    r = __builtin_bit_cast(uint32_t, v) - (134u << 23);
+  } else {
+    const uint32_t odd = (u >> 21) & 1u;
+    u += ((uint32_t)(15 - 127) << 23) + 0xfffffu + odd;
+    r = u >> 21;
+  }
+  return (uint8_t)(r | sign);
+}
+template <> __device__ __forceinline__ e5m2_t from_float<e5m2_t>(float f) { return e5m2_t{float_to_e5m2(f)}; }
+__device__ __forceinline__ float to_float(e5m2_t v) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)((uint16_t)v.bits << 8));
+}
 
 // ---------------------------------------------------------------- vector loads/stores
 template <int BYTES> struct vec_bytes;

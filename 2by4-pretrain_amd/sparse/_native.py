@@ -12,14 +12,14 @@ _LIB_NAME = "lib2by4_gfx950.so"
 _lib = None
 
 # enums of tf24.h
-F32, F16, BF16, E4M3, U8 = 0, 1, 2, 3, 4
+F32, F16, BF16, E4M3, U8, E5M2 = 0, 1, 2, 3, 4, 5
 ROW_MAJOR, COL_MAJOR = 0, 1
 PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
 COMPRESSED_CANONICAL, COMPRESSED_PANEL = 0, 1
 
 _DTYPES = {
-    torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float8_e4m3fn: E4M3,
+    torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float8_e4m3fn: E4M3, torch.float8_e5m2: E5M2,
     torch.uint8: U8, torch.bool: U8, torch.int8: U8,
 }
 

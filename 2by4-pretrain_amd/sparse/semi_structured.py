@@ -29,13 +29,17 @@ _Config = namedtuple("_SEMI_STRUCTURED_SPARSE_CONFIG",
 # semi_structured.py:24-30 of the reference, restricted to what SMFMAC kernels exist for
 _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG = {
     torch.float8_e4m3fn: _Config(10, 32, 128, 16, 16),
+    torch.float8_e5m2: _Config(10, 32, 128, 16, 16),
     torch.float16: _Config(9, 32, 64, 8, 8),
     torch.bfloat16: _Config(9, 32, 64, 8, 8),
 }
 
 
+_FLOAT8 = (torch.float8_e4m3fn, torch.float8_e5m2)
+
+
 def _indices_dtype(values_dtype):
-    if values_dtype == torch.float8_e4m3fn:
+    if values_dtype in _FLOAT8:
         return torch.int32
     if values_dtype in (torch.float16, torch.bfloat16):
         return torch.int16
@@ -125,7 +129,7 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     if kk != k:
         raise RuntimeError(f"inner dimensions do not match: sparse operand has k={k}, dense operand {tuple(dense.shape)}")
     if out_dtype is None:
-        out_dtype = torch.float32 if values.dtype == torch.float8_e4m3fn else values.dtype
+        out_dtype = torch.float32 if values.dtype in _FLOAT8 else values.dtype
     out = torch.empty(out_shape, dtype=out_dtype, device=dense.device)
     if bias is not None:
         bias = bias.to(out_dtype).contiguous()
@@ -286,7 +290,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
         return original_tensor
 
     def _out_dtype(self):
-        return self._FP8_OUT_DTYPE if self.dtype == torch.float8_e4m3fn else None
+        return self._FP8_OUT_DTYPE if self.dtype in _FLOAT8 else None
 
     @classmethod
     def __torch_dispatch__(cls, func, types, args, kwargs) -> Any:
@@ -373,7 +377,7 @@ def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = 
     `mask` (same shape, nonzero = keep) selects explicitly; `MVUE24=True` samples the
     minimum-variance unbiased estimator, taking its uniforms from `rand` (same shape, U[0,1);
     drawn with torch's generator when omitted).  `dtype` is the value dtype of the result
-    (float16, bfloat16 or float8_e4m3fn).  Rows must be a multiple of 32, columns of 64
+    (float16, bfloat16, float8_e4m3fn or float8_e5m2).  Rows must be a multiple of 32, columns of 64
     (128 for float8).  Same signature as the reference's factory (semi_structured.py:575-631)
     plus `rand`.
     """

@@ -42,6 +42,7 @@ typedef enum {
   TF24_F16 = 1,
   TF24_BF16 = 2,
   TF24_E4M3 = 3, /* OCP float8 e4m3fn */
+  TF24_E5M2 = 5, /* OCP float8 e5m2 (IEEE-like: infinities, NaN) */
   TF24_U8 = 4    /* bytes: bool masks (nonzero = kept) */
 } tf24_dtype;
 
@@ -84,8 +85,8 @@ const char* tf24_last_error(void);
  *   mask       [m,k] mask_dtype (U8|F16|BF16|F32), nonzero = kept, same layout, leading dim mask_ld
  *   rand       [m,k] F32 uniforms in [0,1), same layout, leading dim rand_ld; group g of row r
  *              uses rand[r,4g] and rand[r,4g+1]
- *   values     m*k/2 elements of out_dtype (F16|BF16|E4M3) in out_layout
- *   meta       m*k/8 bytes in out_layout (canonical: int16 [m,k/16] for 16-bit values, int32 [m,k/32] for E4M3)
+ *   values     m*k/2 elements of out_dtype (F16|BF16|E4M3|E5M2) in out_layout
+ *   meta       m*k/8 bytes in out_layout (canonical: int16 [m,k/16] for 16-bit values, int32 [m,k/32] for E4M3|E5M2)
  * Shape rules (sparse/semi_structured.py:24-30,188-200): m % 32 == 0, k % 64 == 0 for 16-bit
  * values, k % 128 == 0 for 8-bit values.
  */
@@ -164,7 +165,7 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * Replaces sparse.cutlass.my_sparse_semi_structured_linear
  * (sparse/csrc/mySparseSemiStructuredLinear_cuda.cu:498-817, CUTLASS SparseGemm :61-76),
  * bound at sparse/sparse_semi_structured_linear.py:4-5.
- *   a_values, a_meta  the compressed operand in a_layout; dtype F16|BF16|E4M3 (B has the same dtype)
+ *   a_values, a_meta  the compressed operand in a_layout; dtype F16|BF16|E4M3|E5M2 (B has the same dtype)
  *   b          dense operand, n_dense "columns" j: b_layout TF24_ROW_MAJOR means B is stored
  *              [n_dense, k] (k contiguous, element (k,j) at j*ldb + k: the X of X.W^T);
  *              TF24_COL_MAJOR means stored [k, n_dense] (element (k,j) at k*ldb + j)
@@ -186,7 +187,7 @@ int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype,
 int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense);
 
 /*
- * out[c, r] = in[r, c] for 2-byte (F16|BF16) and 1-byte (E4M3|U8) elements; in [rows, cols] with
+ * out[c, r] = in[r, c] for 2-byte (F16|BF16) and 1-byte (E4M3|E5M2|U8) elements; in [rows, cols] with
  * leading dimension ld_in, out [cols, rows] with ld_out.  No counterpart in the reference (CUTLASS
  * reads either operand layout): it feeds tf24_spmm's fast kernel, which wants the dense operand
  * with k contiguous, when `S @ dense` arrives with a row-major dense (dW = MVUE(dY^T) @ x).

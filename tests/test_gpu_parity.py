@@ -8,7 +8,8 @@ import oracle
 
 pytestmark = pytest.mark.gpu
 
-F16, BF16, F32, E4M3 = torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn
+F16, BF16, F32, E4M3, E5M2 = torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn, torch.float8_e5m2
+FLOAT8 = (E4M3, E5M2)
 
 
 def bits(t):
@@ -44,7 +45,7 @@ def maybe_t(x, col_major):
 # ------------------------------------------------------------------ prune + compress
 @pytest.mark.parametrize("col_major", [False, True])
 @pytest.mark.parametrize("in_dtype", [F16, BF16, F32])
-@pytest.mark.parametrize("out_dtype", [F16, BF16, E4M3])
+@pytest.mark.parametrize("out_dtype", [F16, BF16, E4M3, E5M2])
 @pytest.mark.parametrize("shape", [(32, 128), (96, 320 + 64), (64, 1024)])
 def test_magnitude_compress(cuda, shape, in_dtype, out_dtype, col_major):
     import sparse
@@ -143,7 +144,7 @@ def test_mask_layout_mismatch_is_copied(cuda):
 
 
 @pytest.mark.parametrize("col_major", [False, True])
-@pytest.mark.parametrize("in_dtype,out_dtype", [(BF16, F16), (F16, F16), (F32, BF16), (BF16, E4M3), (F32, E4M3)])
+@pytest.mark.parametrize("in_dtype,out_dtype", [(BF16, F16), (F16, F16), (F32, BF16), (BF16, E4M3), (F32, E4M3), (F32, E5M2)])
 @pytest.mark.parametrize("shape", [(32, 128), (128, 640)])
 def test_mvue_compress(cuda, shape, in_dtype, out_dtype, col_major):
     import sparse
@@ -306,14 +307,14 @@ def _small_ints(shape, seed, lo=-3, hi=4):
     return torch.randint(lo, hi, shape, generator=torch.Generator().manual_seed(seed)).float()
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16, E4M3])
+@pytest.mark.parametrize("dtype", [F16, BF16, E4M3, E5M2])
 @pytest.mark.parametrize("dims", [(32, 128, 16), (64, 256, 40), (96, 384, 200), (160, 1024, 72)])
 def test_spmm_exact_small_integers(cuda, dtype, dims):
     """Small-integer operands: every product and partial sum is exact in float32, so the
     result must EQUAL the dense masked product -- pins operand and index layout."""
     import sparse
     n, k, m = dims
-    if dtype == E4M3 and m % 16:
+    if dtype in FLOAT8 and m % 16:
         m += 8
     w = _small_ints((n, k), 51).to(dtype)
     x = _small_ints((m, k), 52).to(dtype)
@@ -322,7 +323,7 @@ def test_spmm_exact_small_integers(cuda, dtype, dims):
     s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
     out = torch.mm(x.to(cuda), s.t())                      # second operand sparse: x . W^T
     assert out.shape == (m, n)
-    assert out.dtype == (torch.float32 if dtype == E4M3 else dtype)
+    assert out.dtype == (torch.float32 if dtype in FLOAT8 else dtype)
     ref = ref.to(out.dtype).float()                        # the kernel rounds the exact sum once
     assert out.float().cpu().equal(ref)
     # first operand sparse: W . B with B [k, j] row-major (k strided) and as a transposed view
@@ -336,13 +337,13 @@ def test_spmm_exact_small_integers(cuda, dtype, dims):
     assert out4.float().cpu().equal(ref)
 
 
-@pytest.mark.parametrize("dtype,tol", [(F16, 1e-2), (BF16, 1e-2), (E4M3, 5e-2)])
+@pytest.mark.parametrize("dtype,tol", [(F16, 1e-2), (BF16, 1e-2), (E4M3, 5e-2), (E5M2, 5e-2)])
 def test_spmm_random_tolerance(cuda, dtype, tol):
     import sparse
-    n, k, m = 256, 512, 328 if dtype != E4M3 else 336
+    n, k, m = 256, 512, 328 if dtype not in FLOAT8 else 336
     w = randn((n, k), F32, 53, scale=0.02)
     x = randn((m, k), F32, 54)
-    if dtype == E4M3:
+    if dtype in FLOAT8:
         sw, sx = 448.0 / w.abs().max(), 448.0 / x.abs().max()
         wq, xq = (w * sw).to(dtype), (x * sx).to(dtype)
     else:
@@ -390,20 +391,21 @@ def test_dispatch_rules(cuda):
         s + 1
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", [F16, BF16, E4M3, E5M2])
 def test_spmm_tiled_all_operand_positions(cuda, dtype):
     """Shapes large enough for the tiled kernel, with partial tiles: both operand positions, both
     layouts of the dense operand, bias, and the i-major / j-major LDS-staged epilogues."""
     import sparse
-    n, k, m = 352, 640, 296
+    n, k, m = 352, 640, 296 if dtype not in FLOAT8 else 304
+    odt = torch.float32 if dtype in FLOAT8 else dtype           # 8-bit operands return float32
     w = _small_ints((n, k), 61).to(dtype)
     x = _small_ints((m, k), 62).to(dtype)
-    bias = _small_ints((n,), 63).to(dtype)
+    bias = _small_ints((n,), 63).to(odt)
     mask = oracle.prune24_mask(w.float())
     ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
-    ref_b = (ref + bias.float()).to(dtype).float()
-    ref = ref.to(dtype).float()
-    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    ref_b = (ref + bias.float()).to(odt).float()
+    ref = ref.to(odt).float()
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
     xg = x.to(cuda)
     assert torch.mm(xg, s.t()).float().cpu().equal(ref)                          # k contiguous, j-major store
     assert torch.mm(maybe_t(xg, True), s.t()).float().cpu().equal(ref)           # k strided dense operand
