@@ -46,8 +46,45 @@ int launch(const void* values, const void* meta, bool panel, int64_t m, int64_t 
   return check_launch("tf24_decompress");
 }
 
+// Canonical <-> panel storage of a compressed operand.  Per row and panel the 64 value bytes and the
+// KP/8 metadata bytes are the same in both forms, only their place differs: a lane moves 16 value
+// bytes, the first lanes of a row-panel also its metadata.
+__global__ void __launch_bounds__(kThreads)
+repack_kernel(const uint8_t* __restrict__ vin, const uint8_t* __restrict__ min_, int64_t m, int64_t panels, int meta_bytes,
+              bool to_panel, uint8_t* __restrict__ vout, uint8_t* __restrict__ mout) {
+  const int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x;   // 4 lanes per (row, panel), canonical order
+  const int64_t chunk = t >> 2;
+  const int part = (int)(t & 3);
+  if (chunk >= m * panels) return;
+  const int64_t row = chunk / panels, p = chunk - row * panels;
+  const int64_t canon = row * panels + p, panel = p * m + row;
+  const int64_t src = to_panel ? canon : panel, dst = to_panel ? panel : canon;
+  *reinterpret_cast<uint4*>(vout + dst * 64 + part * 16) = *reinterpret_cast<const uint4*>(vin + src * 64 + part * 16);
+  if (part * 8 < meta_bytes)
+    *reinterpret_cast<uint2*>(mout + dst * meta_bytes + part * 8) = *reinterpret_cast<const uint2*>(min_ + src * meta_bytes + part * 8);
+}
+
 }  // namespace
 }  // namespace tf24
+
+extern "C" int tf24_repack(const void* values_in, const void* meta_in, int dtype, int64_t m, int64_t k, int from_layout,
+                           void* values_out, void* meta_out, void* stream) {
+  using namespace tf24;
+  const char* fn = "tf24_repack";
+  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_float8(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
+  const int64_t kp = is_float8(dtype) ? 128 : 64;
+  if (m <= 0 || k <= 0 || k % kp) return fail(TF24_ERR_SHAPE, "%s: k=%lld must be a positive multiple of %lld", fn, (long long)k, (long long)kp);
+  if (from_layout != TF24_COMPRESSED_CANONICAL && from_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, from_layout);
+  if (!values_in || !meta_in || !values_out || !meta_out) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
+  if (values_in == values_out || meta_in == meta_out) return fail(TF24_ERR_ARG, "%s: in-place conversion is not supported", fn);
+  if (((uintptr_t)values_in | (uintptr_t)values_out) % 16 || ((uintptr_t)meta_in | (uintptr_t)meta_out) % 8)
+    return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte and metadata 8-byte aligned", fn);
+  const int64_t panels = k / kp, threads = m * panels * 4;
+  dim3 grid((unsigned)((threads + kThreads - 1) / kThreads));
+  hipLaunchKernelGGL(repack_kernel, grid, dim3(kThreads), 0, (hipStream_t)stream, (const uint8_t*)values_in, (const uint8_t*)meta_in, m, panels,
+                     (int)(kp / 8), from_layout == TF24_COMPRESSED_CANONICAL, (uint8_t*)values_out, (uint8_t*)meta_out);
+  return check_launch(fn);
+}
 
 extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, int layout, int64_t m, int64_t k,
                                void* dense_out, void* stream) {

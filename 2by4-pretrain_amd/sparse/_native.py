@@ -35,6 +35,7 @@ _SIGNATURES = {
     "tf24_prune_compress": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p]),
     "tf24_prune_compress_validate": (_i, [_i, _i, _i64, _i64, _i64, _i, _i, _i, _i64, _i, _i64, _i]),
     "tf24_decompress": (_i, [_p, _i, _p, _i, _i64, _i64, _p, _p]),
+    "tf24_repack": (_i, [_p, _p, _i, _i64, _i64, _i, _p, _p, _p]),
     "tf24_transposable_mask": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _p, _p]),
     "tf24_transposable_mask_validate": (_i, [_i, _i, _i64, _i64, _i64]),
     "tf24_soft_threshold24": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _p, _p]),

@@ -99,8 +99,16 @@ def _compress(original, dtype, MVUE24, mask, rand, panel):
 def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, activation=N.ACT_NONE):
     """sparse_first: out = S @ dense  (S [n,k], dense [k,j])  -> [n, j]
        otherwise   : out = dense @ S^T (dense [j,k])          -> [j, n]"""
-    values, meta = sparse._store_values, sparse._store_meta
+    values, meta, store_layout = sparse._store_values, sparse._store_meta, sparse._store_layout
     n, k = sparse._store_shape
+    # An operand built from canonical values/metadata (the functional entry point) is brought to the
+    # panel form once: the tiled kernel only streams that one.
+    if (store_layout == N.COMPRESSED_CANONICAL and n >= 64 and dense.numel() // k >= 64 and k % _panel_width(values.dtype) == 0):
+        pv, pm = torch.empty_like(values), torch.empty_like(meta)
+        N.check(N.lib().tf24_repack(values.data_ptr(), meta.data_ptr(), N.dtype_code(values.dtype), n, k, N.COMPRESSED_CANONICAL,
+                                    pv.data_ptr(), pm.data_ptr(), N.stream_ptr()))
+        sparse._set_storage(pv, pm, (n, k), N.COMPRESSED_PANEL)
+        values, meta, store_layout = pv, pm, N.COMPRESSED_PANEL
     if dense.dtype != values.dtype:
         raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
     dense = N.as_matrix(dense)
@@ -109,7 +117,7 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     # (`S @ dense` with a row-major dense, e.g. dW = MVUE(dY^T) @ x) one transposing copy of the dense
     # operand is far cheaper than running the general kernel.
     k_strided = (lay == N.ROW_MAJOR) if sparse_first else (lay == N.COL_MAJOR)
-    if k_strided and sparse._store_layout == N.COMPRESSED_PANEL and dense.numel() >= (1 << 16):
+    if k_strided and store_layout == N.COMPRESSED_PANEL and dense.numel() >= (1 << 16):
         v = 16 // dense.element_size()
         row_major = dense if sparse_first else dense.t()          # the view that is row-major: [k, j]
         if row_major.shape[0] % v == 0 and row_major.shape[1] % v == 0:
@@ -138,7 +146,7 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     ws_bytes = N.lib().tf24_spmm_workspace_bytes(N.dtype_code(values.dtype), n, k, j)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dense.device) if ws_bytes else None
     N.check(N.lib().tf24_spmm(
-        values.data_ptr(), meta.data_ptr(), sparse._store_layout, N.dtype_code(values.dtype), n, k,
+        values.data_ptr(), meta.data_ptr(), store_layout, N.dtype_code(values.dtype), n, k,
         dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.dtype_code(out_dtype), c_layout, out.stride(0),
         N.ptr(bias), float(scale), activation, N.ptr(workspace), ws_bytes, N.stream_ptr()))
     return out

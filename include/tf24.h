@@ -111,6 +111,17 @@ int tf24_decompress(const void* values, int dtype, const void* meta, int layout,
                     void* dense_out, void* stream);
 
 /*
+ * Canonical <-> panel storage of a compressed operand (out of place).  The reference keeps one
+ * storage form, the CUTLASS-reordered one made by _sparse_semi_structured_from_dense_triton
+ * (sparse/_semi_structured_conversions.py:1072-1132); a caller holding canonical values and
+ * metadata converts once to the panel form the tiled matmul streams.
+ *   from_layout  the layout of values_in / meta_in; the outputs get the other one
+ *   k % 64 == 0 (16-bit values) / k % 128 == 0 (8-bit)
+ */
+int tf24_repack(const void* values_in, const void* meta_in, int dtype, int64_t m, int64_t k, int from_layout,
+                void* values_out, void* meta_out, void* stream);
+
+/*
  * Transposable 4x4 mask search over the 90 row-and-column 2:4 patterns.
  * Replaces _to_transposable_sparse_semi_structured_kernel and its launcher
  * (sparse/transposable_semi_structured.py:8-47, :50-94) behind TransposableSparse.forward (:198-200).

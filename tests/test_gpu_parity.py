@@ -414,6 +414,9 @@ def test_spmm_tiled_all_operand_positions(cuda, dtype):
     assert torch.addmm(bias.to(cuda), xg, s.t()).float().cpu().equal(ref_b)
     out = sparse.sparse_semi_structured_linear(xg, s, bias=bias.to(cuda), activation="relu")
     assert out.float().cpu().equal(ref_b.clamp_min(0))
+    # canonical values + metadata through the functional entry point: repacked once, same kernel
+    out = sparse.sparse_semi_structured_linear(xg, s.values(), s.indices(), bias=bias.to(cuda))
+    assert out.float().cpu().equal(ref_b)
 
 
 @pytest.mark.parametrize("dims", [(256, 4096, 256), (96, 2048, 520), (352, 12288 // 4, 200)])
@@ -451,3 +454,30 @@ def test_transpose_copy(cuda, dtype, shape):
     out = N.transposed_copy(t.to(cuda))
     assert out.shape == (cols, rows) and out.is_contiguous()
     assert_same(out, t.t().contiguous())
+
+
+@pytest.mark.parametrize("dtype", [F16, E4M3])
+def test_repack_between_canonical_and_panel(cuda, dtype):
+    """tf24_repack on canonical values/metadata must give the bytes the compress kernel writes in
+    panel form, and back."""
+    import sparse
+    from sparse import _native as N
+    m, k = 96, 640
+    w = randn((m, k), F32, 91)
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    assert s._store_layout == N.COMPRESSED_PANEL
+    pv, pm = s._store_values.contiguous(), s._store_meta.contiguous()
+    cv, cm = s.values().contiguous(), s.indices().contiguous()
+    want_v, want_m = oracle.compress24(w, out_dtype=dtype)
+    assert cv.cpu().view(torch.uint8).equal(want_v.view(torch.uint8)) and cm.cpu().equal(want_m)
+    ov, om = torch.empty_like(pv), torch.empty_like(pm)
+    N.check(N.lib().tf24_repack(cv.data_ptr(), cm.data_ptr(), N.dtype_code(dtype), m, k, N.COMPRESSED_CANONICAL,
+                                ov.data_ptr(), om.data_ptr(), N.stream_ptr()))
+    assert ov.view(torch.uint8).equal(pv.view(torch.uint8)) and om.view(torch.uint8).equal(pm.view(torch.uint8))
+    bv, bm = torch.empty_like(cv), torch.empty_like(cm)
+    N.check(N.lib().tf24_repack(pv.data_ptr(), pm.data_ptr(), N.dtype_code(dtype), m, k, N.COMPRESSED_PANEL,
+                                bv.data_ptr(), bm.data_ptr(), N.stream_ptr()))
+    assert bv.view(torch.uint8).equal(cv.view(torch.uint8)) and bm.view(torch.uint8).equal(cm.view(torch.uint8))
+    with pytest.raises(RuntimeError):
+        N.check(N.lib().tf24_repack(cv.data_ptr(), cm.data_ptr(), N.dtype_code(dtype), m, k + 8, N.COMPRESSED_CANONICAL,
+                                    ov.data_ptr(), om.data_ptr(), N.stream_ptr()))
