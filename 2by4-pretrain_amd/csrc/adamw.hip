@@ -42,8 +42,8 @@ adamw_vec(float* __restrict__ p, const G* __restrict__ grad, float* __restrict__
   Pack<float, 4> pv, mv, vv;
   Pack<G, 4> gv;
   Pack<M, 4> mk;
-  pv.load(p + u * 4); mv.load(m + u * 4); vv.load(v + u * 4); gv.load(grad + u * 4);
-  if constexpr (HAS_MASK) mk.load(mask + u * 4);
+  pv.load(p + u * 4); mv.load(m + u * 4); vv.load(v + u * 4); gv.load_stream(grad + u * 4);
+  if constexpr (HAS_MASK) mk.load_stream(mask + u * 4);
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     bool decay = false;

@@ -20,7 +20,7 @@ decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta
     src = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
   }
   Pack<T, 4> v;
-  v.load(values + src * 4);
+  v.load_stream(values + src * 4);
   const uint32_t mb = meta[src];
   Pack<T, 8> out;
 #pragma unroll
@@ -35,7 +35,7 @@ decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta
       if (p1 == (uint32_t)i) out.v[4 * g + i] = v.v[2 * g + 1];
     }
   }
-  out.store(dense + u * 8);
+  out.store_stream(dense + u * 8);
 }
 
 template <typename T>

@@ -52,7 +52,7 @@ dense_op_row(const T* __restrict__ dense, int64_t ld, int64_t m, int64_t k, cons
   if (col8 * 8 >= k) return;
   const int64_t off = row * ld + col8 * 8;
   Pack<T, 8> in, so, mo;
-  in.load(dense + off);
+  in.load_stream(dense + off);
   float r[4] = {0.f, 0.f, 0.f, 0.f};
   if constexpr (OP == OP_MVUE) {
     const float* rp = rnd + row * rand_ld + col8 * 8;
@@ -73,8 +73,8 @@ dense_op_row(const T* __restrict__ dense, int64_t ld, int64_t m, int64_t k, cons
       mo.v[4 * g + i] = keep ? one_of<T>() : zero_of<T>();
     }
   }
-  so.store(sparse + off);
-  if (mask) mo.store(mask + off);
+  so.store_stream(sparse + off);
+  if (mask) mo.store_stream(mask + off);
 }
 
 // Column-major: element (r,c) at c*ld + r.  Lane owns a 4-column x R-row sub-tile (R = 16 bytes of T).
@@ -89,10 +89,10 @@ dense_op_col(const T* __restrict__ dense, int64_t ld, int64_t m, int64_t k, cons
   Pack<T, R> in[4], so[4], mo[4];
   Pack<float, R> rr[2];
 #pragma unroll
-  for (int c = 0; c < 4; c++) in[c].load(dense + (c0 + c) * ld + r0);
+  for (int c = 0; c < 4; c++) in[c].load_stream(dense + (c0 + c) * ld + r0);
   if constexpr (OP == OP_MVUE) {
-    rr[0].load(rnd + (c0 + 0) * rand_ld + r0);
-    rr[1].load(rnd + (c0 + 1) * rand_ld + r0);
+    rr[0].load_stream(rnd + (c0 + 0) * rand_ld + r0);
+    rr[1].load_stream(rnd + (c0 + 1) * rand_ld + r0);
   }
 #pragma unroll
   for (int i = 0; i < R; i++) {
@@ -111,8 +111,8 @@ dense_op_col(const T* __restrict__ dense, int64_t ld, int64_t m, int64_t k, cons
   }
 #pragma unroll
   for (int c = 0; c < 4; c++) {
-    so[c].store(sparse + (c0 + c) * ld + r0);
-    if (mask) mo[c].store(mask + (c0 + c) * ld + r0);
+    so[c].store_stream(sparse + (c0 + c) * ld + r0);
+    if (mask) mo[c].store_stream(mask + (c0 + c) * ld + r0);
   }
 }
 

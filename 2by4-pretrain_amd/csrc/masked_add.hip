@@ -17,8 +17,8 @@ masked_add_vec(G* __restrict__ grad, const P* __restrict__ p, const M* __restric
   Pack<P, 8> pv;
   Pack<M, 8> mk;
   g.load(grad + u * 8);
-  pv.load(p + u * 8);
-  mk.load(mask + u * 8);
+  pv.load_stream(p + u * 8);        // read once; the gradient is read and written: ordinary accesses
+  mk.load_stream(mask + u * 8);
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const float prod = to_float(pv.v[i]) * alpha;

@@ -84,10 +84,10 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
         ounit = row * upr + col8;
       }
       Pack<In, 8> in;
-      in.load(dense + row * ld + col8 * 8);
+      in.load_stream(dense + row * ld + col8 * 8);
       Pack<MaskT, 8> mk;
       float r[4] = {0.f, 0.f, 0.f, 0.f};
-      if constexpr (MODE == TF24_PRUNE_MASK) mk.load(mask + row * mask_ld + col8 * 8);
+      if constexpr (MODE == TF24_PRUNE_MASK) mk.load_stream(mask + row * mask_ld + col8 * 8);
       if constexpr (MODE == TF24_PRUNE_MVUE) {
         const float* rp = rnd + row * rand_ld + col8 * 8;
         float2 ra = *reinterpret_cast<const float2*>(rp);
@@ -106,7 +106,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
         out.v[2 * g + 1] = from_float<Out>(kept_value<MODE>(nib >> 2, x, pr));
         mbyte |= nib << (4 * g);
       }
-      out.store(values + ounit * 4);
+      out.store_stream(values + ounit * 4);
     }
     // 4 adjacent lanes (32 dense columns of one row) -> one metadata dword
     uint32_t w = mbyte;
@@ -142,14 +142,14 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     Pack<MaskT, R> mk[4];
     Pack<float, R> rr[2];
 #pragma unroll
-    for (int c = 0; c < 4; c++) in[c].load(dense + (c0 + c) * ld + r0);
+    for (int c = 0; c < 4; c++) in[c].load_stream(dense + (c0 + c) * ld + r0);
     if constexpr (MODE == TF24_PRUNE_MASK) {
 #pragma unroll
-      for (int c = 0; c < 4; c++) mk[c].load(mask + (c0 + c) * mask_ld + r0);
+      for (int c = 0; c < 4; c++) mk[c].load_stream(mask + (c0 + c) * mask_ld + r0);
     }
     if constexpr (MODE == TF24_PRUNE_MVUE) {
-      rr[0].load(rnd + (c0 + 0) * rand_ld + r0);
-      rr[1].load(rnd + (c0 + 1) * rand_ld + r0);
+      rr[0].load_stream(rnd + (c0 + 0) * rand_ld + r0);
+      rr[1].load_stream(rnd + (c0 + 1) * rand_ld + r0);
     }
 #pragma unroll
     for (int i = 0; i < R; i++) {

@@ -122,7 +122,7 @@ transposable_kernel(const T* __restrict__ dense, int64_t ld, int64_t nmajor4, in
   const int64_t off = bmajor * 4 * ld + bminor * 8;
   Pack<T, 8> in[4];
 #pragma unroll
-  for (int p = 0; p < 4; p++) in[p].load(dense + off + p * ld);
+  for (int p = 0; p < 4; p++) in[p].load_stream(dense + off + p * ld);
   uint32_t mbits[2];
 #pragma unroll
   for (int h = 0; h < 2; h++) {
@@ -150,8 +150,8 @@ transposable_kernel(const T* __restrict__ dense, int64_t ld, int64_t nmajor4, in
         bytes[h] |= (uint32_t)keep << (8 * e);
         out.v[4 * h + e] = keep ? in[p].v[4 * h + e] : T{};
       }
-    *reinterpret_cast<uint2*>(mask_out + off + p * ld) = make_uint2(bytes[0], bytes[1]);
-    if (sparse) out.store(sparse + off + p * ld);
+    *reinterpret_cast<uint2*>(mask_out + off + p * ld) = make_uint2(bytes[0], bytes[1]);   // streaming here costs 15 %
+    if (sparse) out.store_stream(sparse + off + p * ld);
   }
 }
 
