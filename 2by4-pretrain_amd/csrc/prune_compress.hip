@@ -90,9 +90,10 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       if constexpr (MODE == TF24_PRUNE_MASK) mk.load_stream(mask + row * mask_ld + col8 * 8);
       if constexpr (MODE == TF24_PRUNE_MVUE) {
         const float* rp = rnd + row * rand_ld + col8 * 8;
-        float2 ra = *reinterpret_cast<const float2*>(rp);
-        float2 rb = *reinterpret_cast<const float2*>(rp + 4);
-        r[0] = ra.x; r[1] = ra.y; r[2] = rb.x; r[3] = rb.y;
+        Pack<float, 2> ra, rb;                                 // the group's two uniforms; read once
+        ra.load_stream(rp);
+        rb.load_stream(rp + 4);
+        r[0] = ra.v[0]; r[1] = ra.v[1]; r[2] = rb.v[0]; r[3] = rb.v[1];
       }
 #pragma unroll
       for (int g = 0; g < 2; g++) {
