@@ -90,6 +90,10 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
         N.check(lib.tf24_prune_compress(W[i].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MAGNITUDE, None, N.U8, 0,
                                         None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
 
+    def magnitude_canonical(i):
+        N.check(lib.tf24_prune_compress(W[i].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MAGNITUDE, None, N.U8, 0,
+                                        None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_CANONICAL, st))
+
     def mvue(i):
         N.check(lib.tf24_prune_compress(W[i].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MVUE, None, N.U8, 0,
                                         U[i].data_ptr(), k, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
@@ -114,6 +118,8 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
     # algorithmic bytes: every input read once, every output written once
     table = [
         ("magnitude_prune_compress_bf16_to_f16", magnitude, 2 * n + n + n // 8),
+        ("magnitude_prune_compress_bf16_to_f16 (canonical row-major output instead of the matmul's panel layout)",
+         magnitude_canonical, 2 * n + n + n // 8),
         ("mvue24_prune_compress_bf16_u32_to_f16", mvue, 2 * n + 4 * n + n + n // 8),
         ("transposable_mask_select_bf16", transposable, 2 * n + 2 * n + n),
         ("soft_threshold24_bf16", soft, 2 * n + 2 * n + 2 * n),
