@@ -481,3 +481,20 @@ def test_repack_between_canonical_and_panel(cuda, dtype):
     with pytest.raises(RuntimeError):
         N.check(N.lib().tf24_repack(cv.data_ptr(), cm.data_ptr(), N.dtype_code(dtype), m, k + 8, N.COMPRESSED_CANONICAL,
                                     ov.data_ptr(), om.data_ptr(), N.stream_ptr()))
+
+
+@pytest.mark.parametrize("dtype,k", [(F16, 64), (F16, 128), (F16, 192), (F16, 256), (BF16, 320), (E4M3, 128), (E4M3, 256), (E5M2, 384)])
+def test_spmm_tiled_short_k(cuda, dtype, k):
+    """One to five pipeline stages: prologue, steady state and drain of the tiled kernel's stage ring
+    each with fewer stages than the ring holds."""
+    import sparse
+    n, m = 128, 144
+    w = _small_ints((n, k), 93).to(dtype)
+    x = _small_ints((m, k), 94).to(dtype)
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    out = torch.mm(x.to(cuda), s.t())
+    assert out.float().cpu().equal(ref.to(out.dtype).float())
+    out = torch.mm(s, x.to(cuda).t())
+    assert out.float().cpu().equal(ref.t().to(out.dtype).float())
