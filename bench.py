@@ -1,6 +1,6 @@
 """Benchmark of the 2:4 sparse hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|convert]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|train|fp8] [--no-cpu] [--no-convert]
 
 Default workload: BASELINE config 3 -- fp16 2:4 spMM forward  Y[8192,11008] = X[8192,4096] . W^T
 (W[11008,4096] magnitude-pruned along K) plus the transposed product dX[8192,4096] = dY . W with
