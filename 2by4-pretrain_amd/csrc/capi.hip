@@ -77,6 +77,10 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
       if (!has_rand) return fail(TF24_ERR_ARG, "%s: mode MVUE needs a rand tensor", fn);
       if ((rc = check_ld(fn, "rand", layout, rand_ld, m, k))) return rc;
       break;
+    case TF24_PRUNE_MVUE_PACKED:
+      if (!has_rand) return fail(TF24_ERR_ARG, "%s: mode MVUE_PACKED needs a rand tensor", fn);
+      if ((rc = check_ld(fn, "rand", layout, rand_ld, m, k / 2))) return rc;
+      break;
     default:
       return fail(TF24_ERR_ARG, "%s: bad mode %d", fn, mode);
   }

@@ -53,7 +53,8 @@ __global__ void __launch_bounds__(kThreads)
 prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift) {
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift,
+                   bool rand_packed) {
   constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
   const int64_t upr = k >> 3;                             // 8-element units per row
   const int64_t total = m * upr;
@@ -89,11 +90,17 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       float r[4] = {0.f, 0.f, 0.f, 0.f};
       if constexpr (MODE == TF24_PRUNE_MASK) mk.load_stream(mask + row * mask_ld + col8 * 8);
       if constexpr (MODE == TF24_PRUNE_MVUE) {
-        const float* rp = rnd + row * rand_ld + col8 * 8;
-        Pack<float, 2> ra, rb;                                 // the group's two uniforms; read once
-        ra.load_stream(rp);
-        rb.load_stream(rp + 4);
-        r[0] = ra.v[0]; r[1] = ra.v[1]; r[2] = rb.v[0]; r[3] = rb.v[1];
+        if (rand_packed) {                                     // [m, k/2]: the unit's four uniforms are adjacent
+          Pack<float, 4> r4;
+          r4.load_stream(rnd + row * rand_ld + col8 * 4);
+          r[0] = r4.v[0]; r[1] = r4.v[1]; r[2] = r4.v[2]; r[3] = r4.v[3];
+        } else {
+          const float* rp = rnd + row * rand_ld + col8 * 8;
+          Pack<float, 2> ra, rb;                               // the group's two uniforms; read once
+          ra.load_stream(rp);
+          rb.load_stream(rp + 4);
+          r[0] = ra.v[0]; r[1] = ra.v[1]; r[2] = rb.v[0]; r[3] = rb.v[1];
+        }
       }
 #pragma unroll
       for (int g = 0; g < 2; g++) {
@@ -125,7 +132,7 @@ __global__ void __launch_bounds__(kThreads)
 prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel) {
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel, bool rand_packed) {
   constexpr int R = 16 / sizeof(In);
   constexpr int TR = 8 * R;          // tile rows
   constexpr int TC = 128;            // tile columns (32 groups)
@@ -149,8 +156,9 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       for (int c = 0; c < 4; c++) mk[c].load_stream(mask + (c0 + c) * mask_ld + r0);
     }
     if constexpr (MODE == TF24_PRUNE_MVUE) {
-      rr[0].load_stream(rnd + (c0 + 0) * rand_ld + r0);
-      rr[1].load_stream(rnd + (c0 + 1) * rand_ld + r0);
+      const int64_t rc = rand_packed ? c0 >> 1 : c0;           // packed: columns 2g, 2g+1 of a [m, k/2] tensor
+      rr[0].load_stream(rnd + (rc + 0) * rand_ld + r0);
+      rr[1].load_stream(rnd + (rc + 1) * rand_ld + r0);
     }
 #pragma unroll
     for (int i = 0; i < R; i++) {
@@ -227,10 +235,10 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
 
 template <typename In, typename Out, int MODE, typename MaskT>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
-           const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t stream) {
+           const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t stream) {
   if (layout == TF24_ROW_MAJOR) {
     const int64_t per_block = kThreads * kUnroll;
-    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == k);
+    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == (rand_packed ? k / 2 : k));
     const int64_t total = m * (k >> 3);
     dim3 grid((unsigned)((total + per_block - 1) / per_block));
     // lanes per row (log2): 16 lanes read 256 consecutive bytes of bf16 and the four rows of a wave
@@ -242,27 +250,27 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
     }
     hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
                        (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta,
-                       contiguous, panel, lpr_shift);
+                       contiguous, panel, lpr_shift, rand_packed);
   } else {
     constexpr int R = 16 / sizeof(In);
     dim3 grid((unsigned)((k + 127) / 128), (unsigned)((m + 8 * R - 1) / (8 * R)));
     hipLaunchKernelGGL((prune_compress_col<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
-                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel);
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel, rand_packed);
   }
   return check_launch("tf24_prune_compress");
 }
 
 template <typename In, typename Out, int MODE>
 int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int mask_dtype,
-                  int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t s) {
+                  int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
   if constexpr (MODE != TF24_PRUNE_MASK) {
-    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, values, meta, panel, s);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, rand_packed, values, meta, panel, s);
   } else {
     switch (mask_dtype) {
-      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
-      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
-      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
-      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, values, meta, panel, s);
+      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
     }
     return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported mask dtype %d", mask_dtype);
   }
@@ -270,26 +278,27 @@ int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t 
 
 template <typename In, typename Out>
 int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t s) {
+                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
   switch (mode) {
     case TF24_PRUNE_MAGNITUDE:
-      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
     case TF24_PRUNE_MASK:
-      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
     case TF24_PRUNE_MVUE:
-      return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_PRUNE_MVUE_PACKED:
+      return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
   }
   return fail(TF24_ERR_ARG, "tf24_prune_compress: bad mode %d", mode);
 }
 
 template <typename In>
 int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, void* values, void* meta, bool panel, hipStream_t s) {
+                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
   switch (out_dtype) {
-    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
-    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
-    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
-    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported output dtype %d", out_dtype);
 }
@@ -309,11 +318,12 @@ extern "C" int tf24_prune_compress(const void* dense, int in_dtype, int layout, 
   if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
     return fail(TF24_ERR_ARG, "tf24_prune_compress: bad compressed layout %d", out_layout);
   const bool panel = out_layout == TF24_COMPRESSED_PANEL;
+  const bool rand_packed = mode == TF24_PRUNE_MVUE_PACKED;
   hipStream_t s = (hipStream_t)stream;
   switch (in_dtype) {
-    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, values, meta, panel, s);
+    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported input dtype %d", in_dtype);
 }

@@ -83,9 +83,16 @@ def _compress(original, dtype, MVUE24, mask, rand, panel):
     elif MVUE24:
         mode = N.PRUNE_MVUE
         if rand is None:
-            rand = torch.empty_strided(dense.shape, dense.stride(), dtype=torch.float32, device=dense.device).uniform_()
-        if rand.shape != original.shape:
-            raise RuntimeError(f"rand shape {tuple(rand.shape)} does not match tensor shape {tuple(original.shape)}")
+            # only two uniforms per group of four are used: draw [m, n/2] in the dense operand's layout
+            if layout == N.ROW_MAJOR:
+                rand = torch.rand((m, n // 2), dtype=torch.float32, device=dense.device)
+            else:
+                rand = torch.rand((n // 2, m), dtype=torch.float32, device=dense.device).t()
+        if tuple(rand.shape) == (m, n // 2):
+            mode = N.PRUNE_MVUE_PACKED               # group g of a row uses rand[r, 2g], rand[r, 2g+1]
+        elif rand.shape != original.shape:
+            raise RuntimeError(f"rand shape {tuple(rand.shape)} does not match tensor shape {tuple(original.shape)} "
+                               f"(or its packed form {(m, n // 2)})")
         rand_t = N.as_matrix(rand.float(), like=dense)
         rand_ld = N.layout_of(rand_t)[1]
     N.check(N.lib().tf24_prune_compress(

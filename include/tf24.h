@@ -51,7 +51,8 @@ typedef enum { TF24_ROW_MAJOR = 0, TF24_COL_MAJOR = 1 } tf24_layout;
 typedef enum {
   TF24_PRUNE_MAGNITUDE = 0, /* keep the 2 largest |x| per group, ties -> larger index */
   TF24_PRUNE_MASK = 1,      /* keep what a supplied mask says */
-  TF24_PRUNE_MVUE = 2       /* MVUE24 sampling from a supplied U(0,1) tensor */
+  TF24_PRUNE_MVUE = 2,      /* MVUE24 sampling from a supplied U(0,1) tensor of the dense shape */
+  TF24_PRUNE_MVUE_PACKED = 3 /* the same with only the uniforms that are used: a [m, k/2] tensor */
 } tf24_prune_mode;
 
 /* GELU is the exact (erf) form, torch.nn.functional.gelu's default; the reference's epilogues stop at SILU */
@@ -81,10 +82,11 @@ const char* tf24_last_error(void);
  * (sparse/_semi_structured_conversions.py:431-661, :664-1069, launcher :1072-1132),
  * called from SparseSemiStructuredTensor.__init__ (sparse/semi_structured.py:244-245).
  *   dense      [m,k] in_dtype (F32|F16|BF16), (layout, ld)
- *   mode       MAGNITUDE | MASK (mask required) | MVUE (rand required)
+ *   mode       MAGNITUDE | MASK (mask required) | MVUE, MVUE_PACKED (rand required)
  *   mask       [m,k] mask_dtype (U8|F16|BF16|F32), nonzero = kept, same layout, leading dim mask_ld
  *   rand       [m,k] F32 uniforms in [0,1), same layout, leading dim rand_ld; group g of row r
- *              uses rand[r,4g] and rand[r,4g+1]
+ *              uses rand[r,4g] and rand[r,4g+1]; mode MVUE_PACKED: [m,k/2], group g uses
+ *              rand[r,2g] and rand[r,2g+1] (half the bytes to generate and to read)
  *   values     m*k/2 elements of out_dtype (F16|BF16|E4M3|E5M2) in out_layout
  *   meta       m*k/8 bytes in out_layout (canonical: int16 [m,k/16] for 16-bit values, int32 [m,k/32] for E4M3|E5M2)
  * Shape rules (sparse/semi_structured.py:24-30,188-200): m % 32 == 0, k % 64 == 0 for 16-bit

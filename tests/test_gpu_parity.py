@@ -158,6 +158,25 @@ def test_mvue_compress(cuda, shape, in_dtype, out_dtype, col_major):
     assert_same(s.indices(), want_m, "meta")
 
 
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("out_dtype", [F16, E4M3])
+def test_mvue_compress_packed_uniforms(cuda, out_dtype, col_major):
+    """A [m, k/2] uniform tensor holds exactly the uniforms the estimator uses: group g of a row
+    takes columns 2g and 2g+1.  Same result as the full-shape tensor carrying them in columns 4g, 4g+1."""
+    import sparse
+    shape = (64, 384)
+    w = randn(shape, BF16, 25)
+    up = torch.rand((shape[0], shape[1] // 2), generator=torch.Generator().manual_seed(26))
+    full = torch.full(shape, 0.5)
+    full[:, 0::4], full[:, 1::4] = up[:, 0::2], up[:, 1::2]
+    want_v, want_m, _ = oracle.mvue24(w, full, out_dtype=out_dtype)
+    s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major), MVUE24=True, rand=maybe_t(up.to(cuda), col_major), dtype=out_dtype)
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(w.to(cuda), MVUE24=True, rand=up[:, :-8].to(cuda), dtype=out_dtype)
+
+
 def _wide_range(shape, seed):
     """float32 values whose exponents span denormals to 2^60, with zeros, negative zeros and groups
     dominated by one element (sum - a_i rounds to zero): operands the in-range division must hand
