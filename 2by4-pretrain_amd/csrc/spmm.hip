@@ -255,7 +255,7 @@ __device__ __forceinline__ void wait_copies_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <typename T, typename OutT, bool C_JMAJOR, typename C>
+template <typename T, typename OutT, bool C_JMAJOR, typename C, bool B_KSTRIDED>
 __global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
@@ -305,12 +305,25 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   //    (and 256*M_ROW metadata bytes): copy q brings 16 rows x 64 bytes.
   const uint8_t* gb[C::NB];
   const uint8_t* ga[C::NA];
+  // B with k strided (element (k,j) at k*ldb + j, 16-bit types): the stage is kept as [64 k][256 j]
+  // in LDS, copy q brings 2 k-rows x 512 bytes; 16-byte chunks are XOR-swizzled with
+  // ((k & 3) << 1) | ((k >> 3 & 1) << 3) so that the transposing fragment reads below (four k-rows x
+  // 32 bytes per 16 lanes) touch every bank once.  Columns past n_dense re-read the last chunk.
+  constexpr int64_t B_STAGE_ADVANCE_ROWS = B_KSTRIDED ? C::KB / ES : 0;
 #pragma unroll
   for (int q = 0; q < C::NB; q++) {
-    const int row = (wave * C::NB + q) * 8 + (lane >> 3);
-    const int ch = (lane & 7) ^ ((row >> 1) & 7);
-    gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16 + (int64_t)st_begin * C::B_ROW;
+    if constexpr (B_KSTRIDED) {
+      const int krow = (wave * C::NB + q) * 2 + (lane >> 5);
+      const int ch = (lane & 31) ^ (((krow & 3) << 1) | (((krow >> 3) & 1) << 3));
+      const int64_t col = min(j0 + ch * 8, n_dense - 8);
+      gb[q] = b + ((int64_t)st_begin * B_STAGE_ADVANCE_ROWS + krow) * ldb_bytes + col * ES;
+    } else {
+      const int row = (wave * C::NB + q) * 8 + (lane >> 3);
+      const int ch = (lane & 7) ^ ((row >> 1) & 7);
+      gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16 + (int64_t)st_begin * C::B_ROW;
+    }
   }
+  const int64_t b_stage_stride = B_KSTRIDED ? B_STAGE_ADVANCE_ROWS * ldb_bytes : (int64_t)C::B_ROW;
 #pragma unroll
   for (int q = 0; q < C::NA; q++) {
     const int row = (wave * C::NA + q) * 16 + (lane >> 2);
@@ -332,7 +345,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // copy q of this wave for stage st into the stage buffer at LDS byte address `dst`
   const uint32_t smem_at = lds_offset(smem);
   auto issue_one = [&](int q, int st, uint32_t dst) {
-    if (q < C::NB) g2l16(gb[q] + (int64_t)st * C::B_ROW, dst + B_AT + (wave * C::NB + q) * 1024);
+    if (q < C::NB) g2l16(gb[q] + (int64_t)st * b_stage_stride, dst + B_AT + (wave * C::NB + q) * 1024);
     else if (q < C::NB + C::NA) g2l16(ga[q - C::NB] + (int64_t)st * a_stage_stride, dst + (wave * C::NA + q - C::NB) * 1024);
     else g2l4(gm[q - C::NB - C::NA] + (int64_t)st * m_stage_stride, dst + M_AT + (wave * MW + q - C::NB - C::NA) * 256);
   };
@@ -360,6 +373,21 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     for (int h = 0; h < 2; h++) b_off[step][h] = b_row * C::B_ROW + (((step * 4 + h * 2 + lh) ^ b_sw) * 16);
   }
   const int m_off = a_row * M_STEP + lh * (M_STEP / 2);          // inside a step's [row][M_STEP] block
+  // k-strided B: transposing reads (DS_READ_B64_TR_B16).  In a group of 16 lanes, lane i receives
+  // the halfwords i%4 of the source lanes 4e + i/4 (e = 0..3).  Source lane s therefore addresses
+  // k-row k0 + s/4, halfwords 4*(s%4).. of the group's 16 columns, and lane i ends up with
+  // k0..k0+3 of column i: four such reads (k0 = 8*kb + {0, 4, 16, 20}) make one dense fragment.
+  int bt_off[C::TJ];
+  if constexpr (B_KSTRIDED) {
+    const int g16 = lane >> 4, s16 = lane & 15;
+    const int kb = g16 >> 1, jbase = (g16 & 1) * 16;
+    const int swz = ((s16 >> 2) << 1) | (kb << 3);                // (k & 3) << 1 | (k >> 3 & 1) << 3 of the rows read
+#pragma unroll
+    for (int tj = 0; tj < C::TJ; tj++) {
+      const int col = wj * C::WJ + tj * 32 + jbase + (s16 & 3) * 4;  // halfword column in the tile
+      bt_off[tj] = (kb * 8 + (s16 >> 2)) * 512 + (((col >> 3) ^ swz) * 16) + ((col >> 2) & 1) * 8;
+    }
+  }
 
   // ---- main loop: a software pipeline over instruction steps.  While the matrix instructions of a
   // step run from one register set, the fragments of the next step are read from LDS into the
@@ -375,21 +403,31 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   int4v af[2][C::TI];
   int idx[2][C::TI];
   int4v bf[2][C::TJ][2];                         // the two 16-byte halves of a dense fragment
+  typedef short short4v __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) short4v* lds_short4_ptr;
+  short4v bq[2][C::TJ][4];                       // k-strided B: the four 8-byte quarters
   // The reads of a step, in the order the next step's instructions need them: its first row of
   // instructions takes every dense fragment and sparse fragment 0, row r then only needs sparse
   // fragment r.  Read n: dense half-fragment n (fragment n/2, half n%2) for n < 2*TJ, then sparse
   // fragment and index word alternately.
-  constexpr int N_READS = 2 * C::TJ + 2 * C::TI;
+  constexpr int B_READS = (B_KSTRIDED ? 4 : 2) * C::TJ;
+  constexpr int N_READS = B_READS + 2 * C::TI;
   constexpr int READS_PER_ROW = (N_READS + C::TI - 1) / C::TI;
   // `src` is the byte offset of the stage buffer in smem (wave-uniform, changes every stage): the
   // per-lane addresses are formed when needed and fragment offsets ride in the instructions' immediates
   auto read_one = [&](int set, int n, uint32_t src, int step) {
     const uint8_t* base = smem + src;
-    if (n < 2 * C::TJ) {
-      bf[set][n >> 1][n & 1] = *reinterpret_cast<const int4v*>(base + B_AT + b_off[step][n & 1] + (n >> 1) * 32 * C::B_ROW);
+    if (n < B_READS) {
+      if constexpr (B_KSTRIDED) {
+        const int tj = n >> 2, quarter = n & 3;                  // quarter: k0 = 8*kb + {0, 4, 16, 20}
+        const uint8_t* src_q = base + B_AT + bt_off[tj] + step * (32 * 512) + ((quarter & 1) * 4 + (quarter >> 1) * 16) * 512;
+        bq[set][tj][quarter] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(lds_ptr_t)src_q);
+      } else {
+        bf[set][n >> 1][n & 1] = *reinterpret_cast<const int4v*>(base + B_AT + b_off[step][n & 1] + (n >> 1) * 32 * C::B_ROW);
+      }
     } else {
-      const int f = (n - 2 * C::TJ) >> 1;
-      if (((n - 2 * C::TJ) & 1) == 0) af[set][f] = *reinterpret_cast<const int4v*>(base + a_off[step] + f * 32 * C::A_ROW);
+      const int f = (n - B_READS) >> 1;
+      if (((n - B_READS) & 1) == 0) af[set][f] = *reinterpret_cast<const int4v*>(base + a_off[step] + f * 32 * C::A_ROW);
       else if constexpr (ES == 2) idx[set][f] = *reinterpret_cast<const uint16_t*>(base + M_AT + m_off + f * 32 * M_STEP + step * (C::BI * M_STEP));
       else idx[set][f] = *reinterpret_cast<const int*>(base + M_AT + m_off + f * 32 * M_STEP + step * (C::BI * M_STEP));
     }
@@ -404,8 +442,16 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     for (int ti = 0; ti < C::TI; ti++) {
 #pragma unroll
       for (int tj = 0; tj < C::TJ; tj++) {
-        const int4v lo = bf[set][tj][0], hi = bf[set][tj][1];
-        const int8v bfrag = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        int8v bfrag;
+        if constexpr (B_KSTRIDED) {
+          typedef int int2v __attribute__((ext_vector_type(2)));
+          const int2v q0 = __builtin_bit_cast(int2v, bq[set][tj][0]), q1 = __builtin_bit_cast(int2v, bq[set][tj][1]);
+          const int2v q2 = __builtin_bit_cast(int2v, bq[set][tj][2]), q3 = __builtin_bit_cast(int2v, bq[set][tj][3]);
+          bfrag = int8v{q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+        } else {
+          const int4v lo = bf[set][tj][0], hi = bf[set][tj][1];
+          bfrag = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
         acc[ti][tj] = mma32<T>::run(af[set][ti], bfrag, acc[ti][tj], idx[set][ti]);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -643,7 +689,7 @@ int choose_splits(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspac
 }
 
 template <typename T, typename OutT, typename C>
-int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb,
+int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  void* workspace, int64_t workspace_bytes, hipStream_t s) {
   const int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI), tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
@@ -651,14 +697,22 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   const int per_xcd = (tiles_i * tiles_j * splits + 7) / 8;
   dim3 grid((unsigned)(per_xcd * 8));
   const bool jm = c_layout == TF24_COL_MAJOR;
-  if (jm)
-    hipLaunchKernelGGL((spmm_pipe<T, OutT, true, C>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
-                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j,
-                       splits, (float*)workspace);
-  else
-    hipLaunchKernelGGL((spmm_pipe<T, OutT, false, C>), grid, dim3(C::THREADS), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
-                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j,
-                       splits, (float*)workspace);
+  auto launch = [&](auto c_jmajor, auto b_kstrided) {
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value>), grid, dim3(C::THREADS), 0, s,
+                       (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                       (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
+  };
+  bool kstrided = false;
+  if constexpr (sizeof(T) == 2) kstrided = b_layout == TF24_COL_MAJOR;
+  if (kstrided) {
+    if constexpr (sizeof(T) == 2) {
+      if (jm) launch(std::true_type{}, std::true_type{});
+      else launch(std::false_type{}, std::true_type{});
+    }
+  } else {
+    if (jm) launch(std::true_type{}, std::false_type{});
+    else launch(std::false_type{}, std::false_type{});
+  }
   if (splits > 1) {
     dim3 rgrid((unsigned)(tiles_i * tiles_j), 8);
     if (jm)
@@ -691,11 +745,12 @@ template <typename T>
 int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout,
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  void* workspace, int64_t workspace_bytes, hipStream_t s) {
-  if (panel && b_layout == TF24_ROW_MAJOR && n_sparse >= 64 && n_dense >= 64) {
+  // the tiled kernel reads a k-strided dense operand through transposing LDS reads (16-bit types only)
+  if (panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64 && n_dense >= 64) {
     switch (out_dtype) {
-      case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
-      case TF24_BF16: return launch_tiled<T, bf16_t, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
-      case TF24_F32: return launch_tiled<T, float, TiledCfg>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_BF16: return launch_tiled<T, bf16_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_F32: return launch_tiled<T, float, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     }
   }
   switch (out_dtype) {

@@ -120,11 +120,12 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
         raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
     dense = N.as_matrix(dense)
     lay, ld = N.layout_of(dense)
-    # The tiled kernel wants the dense operand with k contiguous.  When k is the strided dimension
-    # (`S @ dense` with a row-major dense, e.g. dW = MVUE(dY^T) @ x) one transposing copy of the dense
+    # When k is the strided dimension of the dense operand (`S @ dense` with a row-major dense, e.g.
+    # dW = MVUE(dY^T) @ x) the tiled kernel reads 16-bit operands as they are, transposing while it
+    # loads fragments.  For 8-bit operands it wants k contiguous: one transposing copy of the dense
     # operand is far cheaper than running the general kernel.
     k_strided = (lay == N.ROW_MAJOR) if sparse_first else (lay == N.COL_MAJOR)
-    if k_strided and store_layout == N.COMPRESSED_PANEL and dense.numel() >= (1 << 16):
+    if k_strided and dense.element_size() == 1 and store_layout == N.COMPRESSED_PANEL and dense.numel() >= (1 << 16):
         v = 16 // dense.element_size()
         row_major = dense if sparse_first else dense.t()          # the view that is row-major: [k, j]
         if row_major.shape[0] % v == 0 and row_major.shape[1] % v == 0:

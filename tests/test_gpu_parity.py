@@ -517,3 +517,23 @@ def test_spmm_tiled_short_k(cuda, dtype, k):
     assert out.float().cpu().equal(ref.to(out.dtype).float())
     out = torch.mm(s, x.to(cuda).t())
     assert out.float().cpu().equal(ref.t().to(out.dtype).float())
+    out = torch.mm(s, x.to(cuda).t().contiguous())                                 # k strided: transposing fragment reads
+    assert out.float().cpu().equal(ref.t().to(out.dtype).float())
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_spmm_tiled_k_strided_padded_rows(cuda, dtype):
+    """`S @ dense` with the dense operand a column slice of a wider row-major matrix: k is the strided
+    dimension, rows are longer than the columns used, and the last column tile is partial."""
+    import sparse
+    n, k, j, ld = 320, 448, 520, 776
+    w = _small_ints((n, k), 95).to(dtype)
+    wide = _small_ints((k, ld), 96).to(dtype)
+    x = wide[:, 8:8 + j]                                                            # [k, j], row pitch ld, 16-byte aligned start
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.t().float(), torch.where(mask, w.float(), torch.zeros(()))).t()   # [n, j]
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    xg = wide.to(cuda)[:, 8:8 + j]
+    assert not xg.is_contiguous()
+    out = torch.mm(s, xg)
+    assert out.float().cpu().equal(ref.to(dtype).float())
