@@ -87,3 +87,21 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
   if (has_mask && has_rand) return fail(TF24_ERR_ARG, "%s: using MVUE24 with mask is not supported", fn);
   return TF24_OK;
 }
+
+extern "C" int tf24_prune_compress_dual_validate(int in_dtype, int64_t ld, int64_t m, int64_t k, int mask_dtype,
+                                                 int64_t mask_ld, int out_dtype, int out_layout) {
+  const char* fn = "tf24_prune_compress_dual";
+  if (!is_float_dtype(in_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
+  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && !is_float8(out_dtype))
+    return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
+  if (!is_mask_dtype(mask_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported mask dtype %d", fn, mask_dtype);
+  if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
+    return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, out_layout);
+  const int64_t unit = is_float8(out_dtype) ? 128 : 64;
+  if (m < unit || m % unit || k < unit || k % unit)
+    return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld) is not supported: both dimensions must be >= and a multiple of %lld",
+                fn, (long long)m, (long long)k, (long long)unit);
+  int rc = check_ld(fn, "dense", TF24_ROW_MAJOR, ld, m, k);
+  if (rc) return rc;
+  return check_ld(fn, "mask", TF24_ROW_MAJOR, mask_ld, m, k);
+}

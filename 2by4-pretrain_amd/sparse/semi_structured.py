@@ -22,7 +22,7 @@ import torch
 
 from . import _native as N
 
-__all__ = ["SparseSemiStructuredTensor", "to_sparse_semi_structured"]
+__all__ = ["SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair"]
 
 _Config = namedtuple("_SEMI_STRUCTURED_SPARSE_CONFIG",
                      "compression_factor sparse_min_rows sparse_min_cols dense_min_rows dense_min_cols")
@@ -400,3 +400,39 @@ def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = 
     return SparseSemiStructuredTensor(
         original_tensor, original_shape=original_tensor.shape, transposed=transposed,
         MVUE24=MVUE24, mask=mask, dtype=dtype, rand=rand)
+
+
+def to_sparse_semi_structured_pair(original_tensor: torch.Tensor, mask: torch.Tensor,
+                                   dtype: torch.dtype = torch.float16):
+    """(to_sparse_semi_structured(w, mask=mask, dtype=dtype), to_sparse_semi_structured(w.T, mask=mask.T, dtype=dtype))
+    from one pass over w and mask: the two compressed copies a transposable-mask training layer
+    rebuilds every optimizer step (README.md:165-166).  Both results are bit-identical to the
+    separate calls.  w [m, k] row-major, both dimensions a multiple of 64 (128 for float8); with
+    any other input the two separate conversions run instead."""
+    w = original_tensor
+    if not w.is_cuda or w.dim() != 2 or dtype not in _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG or mask is None:
+        return (to_sparse_semi_structured(w, mask=mask, dtype=dtype), to_sparse_semi_structured(w.T, mask=mask.T, dtype=dtype))
+    m, k = w.shape
+    unit = _panel_width(dtype)
+    if mask.dtype == torch.bool:
+        mask = mask.view(torch.uint8)
+    lay_w, lay_m = N.layout_of(w), N.layout_of(mask) if mask.dim() == 2 and mask.shape == w.shape else None
+    fits = (m >= unit and k >= unit and m % unit == 0 and k % unit == 0 and w.dtype in (torch.float32, torch.float16, torch.bfloat16)
+            and lay_w is not None and lay_m is not None and lay_w[0] == N.ROW_MAJOR and lay_m[0] == N.ROW_MAJOR
+            and lay_w[1] % 8 == 0 and lay_m[1] % 8 == 0 and w.data_ptr() % 16 == 0 and mask.data_ptr() % 16 == 0
+            and mask.dtype in N._DTYPES and SparseSemiStructuredTensor._PANEL_LAYOUT)
+    if not fits:
+        return (to_sparse_semi_structured(w, mask=mask, dtype=dtype), to_sparse_semi_structured(w.T, mask=mask.T, dtype=dtype))
+    cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[dtype]
+    per = w.nelement() * cfg.compression_factor // 16
+    buf = torch.empty((2 * per,), dtype=dtype, device=w.device)          # [values | meta | values_t | meta_t]
+    half = m * k // 2
+    values, meta = buf[:half], buf[half:per].view(_indices_dtype(dtype))
+    values_t, meta_t = buf[per:per + half], buf[per + half:].view(_indices_dtype(dtype))
+    N.check(N.lib().tf24_prune_compress_dual(
+        w.data_ptr(), N.dtype_code(w.dtype), lay_w[1], m, k, mask.data_ptr(), N.dtype_code(mask.dtype), lay_m[1],
+        values.data_ptr(), meta.data_ptr(), values_t.data_ptr(), meta_t.data_ptr(),
+        N.dtype_code(dtype), N.COMPRESSED_PANEL, N.stream_ptr()))
+    s = SparseSemiStructuredTensor._from_storage(values, meta, (m, k), N.COMPRESSED_PANEL, torch.Size((m, k)), False)
+    s_t = SparseSemiStructuredTensor._from_storage(values_t, meta_t, (k, m), N.COMPRESSED_PANEL, torch.Size((k, m)), False)
+    return s, s_t

@@ -15,7 +15,7 @@ import torch.nn.functional as F
 from torch import autograd, nn
 from torch.amp import custom_bwd, custom_fwd
 
-from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured
+from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair
 from .transposable_semi_structured import TransposableSparse
 
 __all__ = ["SparseLinearTranspose", "sparse_linear_transpose"]
@@ -76,8 +76,9 @@ class SparseLinearTranspose(nn.Linear):
             if w.counter % w.freq == 0 and w.cnt == 0:
                 _, w.mask = self.transposable_sparse(w)
             if w.cnt == 0:
-                w.weight_sparse = to_sparse_semi_structured(w, mask=w.mask, dtype=torch.float16)
-                w.weight_sparse_T = to_sparse_semi_structured(w.T, mask=w.mask.T, dtype=torch.float16)
+                # = to_sparse_semi_structured(w, mask=w.mask), to_sparse_semi_structured(w.T, mask=w.mask.T)
+                # (README.md:165-166), from one read of w and the mask
+                w.weight_sparse, w.weight_sparse_T = to_sparse_semi_structured_pair(w, w.mask, dtype=torch.float16)
             with torch.autocast(device_type='cuda', dtype=torch.float16):
                 x = sparse_linear_transpose.apply(x, w, w.weight_sparse, w.weight_sparse_T, self.bias)
         if self.training:

@@ -112,6 +112,14 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
         N.check(lib.tf24_prune_compress(P[i].data_ptr(), N.F32, N.ROW_MAJOR, k, m, k, N.PRUNE_MASK, bmask[i].data_ptr(), N.U8, k,
                                         None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
 
+    values_t = [torch.empty(k, m // 2, dtype=torch.float16, device=dev) for _ in range(2)]
+    meta_t = [torch.empty(k, m // 16, dtype=torch.int16, device=dev) for _ in range(2)]
+
+    def mask_compress_pair(i):
+        N.check(lib.tf24_prune_compress_dual(P[i].data_ptr(), N.F32, k, m, k, bmask[i].data_ptr(), N.U8, k,
+                                             values[i].data_ptr(), meta[i].data_ptr(), values_t[i % 2].data_ptr(),
+                                             meta_t[i % 2].data_ptr(), N.F16, N.COMPRESSED_PANEL, st))
+
     def copy(i):
         sp[i].copy_(W[i])
 
@@ -125,6 +133,8 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
         ("soft_threshold24_bf16", soft, 2 * n + 2 * n + 2 * n),
         ("masked_add_f32", decay, 4 * n + 4 * n + 4 * n + n),
         ("mask_prune_compress_f32_to_f16", mask_compress, 4 * n + n + n + n // 8),
+        ("mask_prune_compress_W_and_WT_f32_to_f16 (both compressed copies from one read)", mask_compress_pair,
+         4 * n + n + 2 * (n + n // 8)),
         ("device_copy_bf16 (practical HBM ceiling)", copy, 4 * n),
     ]
     out = []

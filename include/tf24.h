@@ -97,6 +97,31 @@ int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld,
                         const float* rand, int64_t rand_ld,
                         void* values, int out_dtype, void* meta, int out_layout, void* stream);
 
+/*
+ * Mask-driven 2:4 compression of W and of W^T from ONE read of W and of the mask:
+ *   (values, meta)      = tf24_prune_compress(W   [m,k] row-major,          mode MASK, mask)
+ *   (values_t, meta_t)  = tf24_prune_compress(W^T [k,m] (W read by columns), mode MASK, mask^T)
+ * bit for bit.  Replaces the pair of conversions the training layer issues once per optimizer step,
+ *   to_sparse_semi_structured(w, mask=w.mask) and to_sparse_semi_structured(w.T, mask=w.mask.T)
+ * (README.md:165-166; each one the `PRUNE == 'mask'` branch of
+ * sparse/_semi_structured_conversions.py:517-533), which read W and the mask twice.
+ *   dense    [m,k] row-major, leading dimension ld; F32|F16|BF16
+ *   mask     [m,k] row-major, leading dimension mask_ld; U8 (bool) or F32|F16|BF16, nonzero = keep.
+ *            Any mask is accepted (groups with other than two kept elements follow the 16-row
+ *            table in either direction); a transposable mask makes both results exact 2:4 copies.
+ *   values, meta      m*k/2 elements of out_dtype and m*k/8 bytes: W compressed along k
+ *   values_t, meta_t  the same sizes: W^T [k,m] compressed along m
+ *   out_layout        TF24_COMPRESSED_CANONICAL or TF24_COMPRESSED_PANEL, for both results
+ * Shape rules: both directions must satisfy tf24_prune_compress's, so m and k are multiples of 64
+ * for 16-bit values and of 128 for 8-bit values.
+ */
+int tf24_prune_compress_dual(const void* dense, int in_dtype, int64_t ld, int64_t m, int64_t k,
+                             const void* mask, int mask_dtype, int64_t mask_ld,
+                             void* values, void* meta, void* values_t, void* meta_t,
+                             int out_dtype, int out_layout, void* stream);
+int tf24_prune_compress_dual_validate(int in_dtype, int64_t ld, int64_t m, int64_t k, int mask_dtype, int64_t mask_ld,
+                                      int out_dtype, int out_layout);
+
 /* The argument checks of tf24_prune_compress without touching the GPU (pointers are only
  * tested for NULL-ness through the has_* flags). Host only. */
 int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld, int64_t m, int64_t k, int mode,
@@ -202,8 +227,9 @@ int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_
 /*
  * out[c, r] = in[r, c] for 2-byte (F16|BF16) and 1-byte (E4M3|E5M2|U8) elements; in [rows, cols] with
  * leading dimension ld_in, out [cols, rows] with ld_out.  No counterpart in the reference (CUTLASS
- * reads either operand layout): it feeds tf24_spmm's fast kernel, which wants the dense operand
- * with k contiguous, when `S @ dense` arrives with a row-major dense (dW = MVUE(dY^T) @ x).
+ * reads either operand layout): it feeds tf24_spmm's fast kernel, which wants an 8-bit dense operand
+ * with k contiguous, when `S @ dense` arrives with a row-major dense (16-bit operands are read
+ * k-strided by the fast kernel itself and need no copy).
  * rows, cols and leading dimensions must be multiples of 16 bytes worth of elements.
  */
 int tf24_transpose(const void* in, int dtype, int64_t ld_in, int64_t rows, int64_t cols, void* out, int64_t ld_out,

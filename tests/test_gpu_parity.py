@@ -130,6 +130,78 @@ def test_mask_compress(cuda, in_dtype, out_dtype, mask_dtype, col_major):
     assert_same(s.indices(), want_m, "meta")
 
 
+@pytest.mark.parametrize("mask_dtype", [torch.bool, BF16, F32])
+@pytest.mark.parametrize("in_dtype,out_dtype,shape", [
+    (F32, F16, (64, 64)), (F32, F16, (192, 320)), (F16, F16, (128, 448)), (BF16, BF16, (320, 128)),
+    (F32, E4M3, (128, 384)), (BF16, E5M2, (256, 128))])
+def test_mask_compress_pair(cuda, in_dtype, out_dtype, mask_dtype, shape):
+    """W and W^T compressed from one read: each result must carry the bytes of the separate
+    conversion of w / w.T (oracle), for transposable masks and for invalid groups."""
+    import sparse
+    from sparse import _native as N
+    w = randn(shape, in_dtype, 15)
+    _, mask = oracle.transposable_mask(w.float())
+    g = torch.Generator().manual_seed(16)
+    mask[:8] = torch.rand(8, shape[1], generator=g) < 0.5        # groups with 0..4 kept elements, both directions
+    mask = mask.to(mask_dtype)
+    want_v, want_m = oracle.compress24(w, mask=mask, out_dtype=out_dtype)
+    want_vt, want_mt = oracle.compress24(w.t().contiguous(), mask=mask.t().contiguous(), out_dtype=out_dtype)
+    s, s_t = sparse.to_sparse_semi_structured_pair(w.to(cuda), mask.to(cuda), dtype=out_dtype)
+    assert s.shape == shape and s_t.shape == shape[::-1]
+    assert s._store_layout == N.COMPRESSED_PANEL and s_t._store_layout == N.COMPRESSED_PANEL
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+    assert_same(s_t.values(), want_vt, "values of the transpose")
+    assert_same(s_t.indices(), want_mt, "meta of the transpose")
+    # canonical output through the C entry point, with padded rows of the dense matrix and the mask
+    m, k = shape
+    wide = torch.zeros((m, k + 24), dtype=in_dtype, device=cuda)
+    wide[:, 8:8 + k] = w.to(cuda)
+    mk = mask.to(cuda)
+    mk = mk.view(torch.uint8) if mk.dtype == torch.bool else mk
+    mwide = torch.zeros((m, k + 16), dtype=mk.dtype, device=cuda)
+    mwide[:, 16:] = mk
+    wv, mv = wide[:, 8:8 + k], mwide[:, 16:]
+    idt = torch.int32 if out_dtype in FLOAT8 else torch.int16
+    cv = torch.empty((m, k // 2), dtype=out_dtype, device=cuda)
+    cvt = torch.empty((k, m // 2), dtype=out_dtype, device=cuda)
+    cm = torch.empty((m, k // 8), dtype=torch.uint8, device=cuda)
+    cmt = torch.empty((k, m // 8), dtype=torch.uint8, device=cuda)
+    N.check(N.lib().tf24_prune_compress_dual(
+        wv.data_ptr(), N.dtype_code(in_dtype), wv.stride(0), m, k, mv.data_ptr(), N.dtype_code(mv.dtype), mv.stride(0),
+        cv.data_ptr(), cm.data_ptr(), cvt.data_ptr(), cmt.data_ptr(), N.dtype_code(out_dtype), N.COMPRESSED_CANONICAL, N.stream_ptr()))
+    assert_same(cv, want_v)
+    assert_same(cm.view(idt), want_m)
+    assert_same(cvt, want_vt)
+    assert_same(cmt.view(idt), want_mt)
+
+
+def test_mask_compress_pair_falls_back_and_rejects(cuda):
+    """Shapes only one direction supports run the two separate conversions (and raise where those
+    raise); the C entry point refuses them."""
+    import sparse
+    from sparse import _native as N
+    w = randn((96, 128), F16, 17)                               # 96 rows: fine for w, not for w.T (needs % 64)
+    mask = oracle.prune24_mask(w)
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured_pair(w.to(cuda), mask.to(cuda))
+    wt = randn((128, 192), F16, 18).t()                         # column-major input: separate conversions, same bytes
+    _, mask = oracle.transposable_mask(wt.contiguous().float())
+    s, s_t = sparse.to_sparse_semi_structured_pair(wt.to(cuda), mask.to(cuda))
+    want_v, want_m = oracle.compress24(wt.contiguous(), mask=mask)
+    want_vt, want_mt = oracle.compress24(wt.t().contiguous(), mask=mask.t().contiguous())
+    assert_same(s.values(), want_v)
+    assert_same(s.indices(), want_m)
+    assert_same(s_t.values(), want_vt)
+    assert_same(s_t.indices(), want_mt)
+    lib = N.lib()
+    assert lib.tf24_prune_compress_dual_validate(N.F16, 128, 96, 128, N.U8, 128, N.F16, N.COMPRESSED_PANEL) != 0
+    assert lib.tf24_prune_compress_dual_validate(N.F16, 128, 128, 128, N.U8, 128, N.E4M3, N.COMPRESSED_PANEL) == 0
+    assert lib.tf24_prune_compress_dual_validate(N.F16, 64, 128, 64, N.U8, 64, N.E4M3, N.COMPRESSED_PANEL) != 0
+    assert lib.tf24_prune_compress_dual_validate(N.F16, 120, 128, 128, N.U8, 128, N.F16, N.COMPRESSED_PANEL) != 0   # ld < k
+    assert lib.tf24_prune_compress_dual_validate(N.U8, 128, 128, 128, N.U8, 128, N.F16, N.COMPRESSED_PANEL) != 0
+
+
 def test_mask_layout_mismatch_is_copied(cuda):
     import sparse
     w = randn((64, 128), F16, 14)

@@ -95,6 +95,22 @@ def test_transposable_and_spmm_validators(native):
     assert sp(N.F16, 32, 64, 8, act=5) == -5 and sp(N.F16, 32, 64, 8, bl=3) == -5
 
 
+def test_dual_compress_validator(native):
+    """Both W [m,k] and W^T [k,m] must be compressible: m and k multiples of 64 (128 for 8-bit values)."""
+    lib, N = native.lib(), native
+    dual = lambda m, k, **kw: lib.tf24_prune_compress_dual_validate(
+        kw.get("dt", N.F32), kw.get("ld", k), m, k, kw.get("mdt", N.U8), kw.get("mld", k), kw.get("out", N.F16),
+        kw.get("lay", N.COMPRESSED_PANEL))
+    assert dual(64, 64) == 0 and dual(3072, 768) == 0 and dual(768, 3072, out=N.BF16, lay=N.COMPRESSED_CANONICAL) == 0
+    assert dual(128, 256, out=N.E4M3) == 0 and dual(128, 256, out=N.E5M2, mdt=N.F32) == 0
+    assert dual(96, 128) == -1 and dual(128, 96) == -1 and dual(32, 64) == -1
+    assert dual(64, 128, out=N.E4M3) == -1 and dual(128, 192, out=N.E4M3) == -1
+    assert dual(64, 64, dt=N.U8) == -2 and dual(64, 64, out=N.F32) == -2 and dual(64, 64, mdt=N.E4M3) == -2
+    assert dual(64, 64, ld=56) == -3 and dual(64, 64, mld=68) == -3
+    assert dual(64, 64, lay=2) == -5
+    assert b"tf24_prune_compress_dual" in lib.tf24_last_error()
+
+
 def test_python_api_rejects_cpu_tensors(native):
     import sparse
     with pytest.raises(RuntimeError, match="Only CUDA tensors"):
