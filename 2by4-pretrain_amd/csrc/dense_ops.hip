@@ -47,8 +47,10 @@ template <typename T, int OP>
 __global__ void __launch_bounds__(kThreads)
 dense_op_row(const T* __restrict__ dense, int64_t ld, int64_t m, int64_t k, const float* __restrict__ rnd, int64_t rand_ld,
              T* __restrict__ sparse, T* __restrict__ mask) {
-  const int64_t col8 = (int64_t)blockIdx.y * kThreads + threadIdx.x;
-  const int64_t row = blockIdx.x;
+  // blocks are numbered along the row first: blocks that run together read neighbouring pieces of one row
+  const uint32_t chunks = (uint32_t)((k / 8 + kThreads - 1) / kThreads);
+  const int64_t row = blockIdx.x / chunks;
+  const int64_t col8 = (int64_t)(blockIdx.x - (uint32_t)row * chunks) * kThreads + threadIdx.x;
   if (col8 * 8 >= k) return;
   const int64_t off = row * ld + col8 * 8;
   Pack<T, 8> in, so, mo;
@@ -84,8 +86,11 @@ __global__ void __launch_bounds__(kThreads)
 dense_op_col(const T* __restrict__ dense, int64_t ld, int64_t m, int64_t k, const float* __restrict__ rnd, int64_t rand_ld,
              T* __restrict__ sparse, T* __restrict__ mask) {
   constexpr int R = 16 / sizeof(T);
-  const int64_t r0 = ((int64_t)blockIdx.y * kThreads + threadIdx.x) * R;
-  const int64_t c0 = (int64_t)blockIdx.x * 4;
+  // blocks are numbered along the contiguous (row) dimension first
+  const uint32_t chunks = (uint32_t)((m / R + kThreads - 1) / kThreads);
+  const int64_t grp = blockIdx.x / chunks;
+  const int64_t r0 = ((int64_t)(blockIdx.x - (uint32_t)grp * chunks) * kThreads + threadIdx.x) * R;
+  const int64_t c0 = grp * 4;
   if (r0 >= m) return;
   Pack<T, R> in[4], so[4], mo[4];
   Pack<float, R> rr[2];
@@ -121,11 +126,11 @@ template <typename T, int OP>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const float* rnd, int64_t rand_ld,
            void* sparse, void* mask, hipStream_t s, const char* fn) {
   if (layout == TF24_ROW_MAJOR) {
-    dim3 grid((unsigned)m, (unsigned)((k / 8 + kThreads - 1) / kThreads));   // x: row, y: column chunk
+    dim3 grid((unsigned)(m * ((k / 8 + kThreads - 1) / kThreads)));
     hipLaunchKernelGGL((dense_op_row<T, OP>), grid, dim3(kThreads), 0, s, (const T*)dense, ld, m, k, rnd, rand_ld, (T*)sparse, (T*)mask);
   } else {
     constexpr int R = 16 / sizeof(T);
-    dim3 grid((unsigned)(k / 4), (unsigned)((m / R + kThreads - 1) / kThreads));   // x: group, y: row chunk
+    dim3 grid((unsigned)((k / 4) * ((m / R + kThreads - 1) / kThreads)));
     hipLaunchKernelGGL((dense_op_col<T, OP>), grid, dim3(kThreads), 0, s, (const T*)dense, ld, m, k, rnd, rand_ld, (T*)sparse, (T*)mask);
   }
   return check_launch(fn);

@@ -68,8 +68,9 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     int64_t row = 0, col8 = 0, ounit = 0;
     if (panel) {
       const int rpi = kThreads >> lpr_shift;                 // rows per iteration
-      row = (int64_t)blockIdx.x * (kUnroll * rpi) + it * rpi + (threadIdx.x >> lpr_shift);
-      col8 = ((int64_t)blockIdx.y << lpr_shift) + (threadIdx.x & ((1 << lpr_shift) - 1));
+      // blocks that run together (consecutive blockIdx.x) read neighbouring column ranges of the same rows
+      row = (int64_t)blockIdx.y * (kUnroll * rpi) + it * rpi + (threadIdx.x >> lpr_shift);
+      col8 = ((int64_t)blockIdx.x << lpr_shift) + (threadIdx.x & ((1 << lpr_shift) - 1));
       live = col8 < upr;                                   // m is a multiple of 32
     }
     if (live) {
@@ -143,7 +144,8 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
 
   const int tid = threadIdx.x;
   const int rchunk = tid & 7, grp = tid >> 3;           // 8 row chunks x 32 groups
-  const int64_t row0 = (int64_t)blockIdx.y * TR, col0 = (int64_t)blockIdx.x * TC;
+  // consecutive blockIdx.x walk the contiguous (row) dimension of the column-major input
+  const int64_t row0 = (int64_t)blockIdx.x * TR, col0 = (int64_t)blockIdx.y * TC;
   const int64_t r0 = row0 + rchunk * R, c0 = col0 + grp * 4;
   if (r0 < m && c0 < k) {
     Pack<In, R> in[4];
@@ -246,14 +248,14 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
     const int lpr_shift = m % (kUnroll * (kThreads >> 4)) == 0 ? 4 : 5;
     if (panel) {
       const int rows_per_block = kUnroll * (kThreads >> lpr_shift), units_per_block = 1 << lpr_shift;
-      grid = dim3((unsigned)(m / rows_per_block), (unsigned)(((k >> 3) + units_per_block - 1) / units_per_block));
+      grid = dim3((unsigned)(((k >> 3) + units_per_block - 1) / units_per_block), (unsigned)(m / rows_per_block));
     }
     hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
                        (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta,
                        contiguous, panel, lpr_shift, rand_packed);
   } else {
     constexpr int R = 16 / sizeof(In);
-    dim3 grid((unsigned)((k + 127) / 128), (unsigned)((m + 8 * R - 1) / (8 * R)));
+    dim3 grid((unsigned)((m + 8 * R - 1) / (8 * R)), (unsigned)((k + 127) / 128));
     hipLaunchKernelGGL((prune_compress_col<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
                        (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel, rand_packed);
   }

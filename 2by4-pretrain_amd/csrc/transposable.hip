@@ -116,8 +116,11 @@ transposable_kernel(const T* __restrict__ dense, int64_t ld, int64_t nmajor4, in
   // "major" = the strided dimension in memory, "minor" = the contiguous one.  A lane owns two
   // adjacent 4 x 4 blocks (8 contiguous elements of 4 lines): 16-byte loads and stores for 16-bit
   // types, 8-byte mask stores.
-  const int64_t bminor = (int64_t)blockIdx.y * kThreads + threadIdx.x;
-  const int64_t bmajor = blockIdx.x;
+  // blocks are numbered along the contiguous dimension first: blocks that run together read
+  // neighbouring pieces of the same four lines
+  const uint32_t chunks = (uint32_t)((nminor8 + kThreads - 1) / kThreads);
+  const int64_t bmajor = blockIdx.x / chunks;
+  const int64_t bminor = (int64_t)(blockIdx.x - (uint32_t)bmajor * chunks) * kThreads + threadIdx.x;
   if (bminor >= nminor8) return;
   const int64_t off = bmajor * 4 * ld + bminor * 8;
   Pack<T, 8> in[4];
@@ -158,7 +161,7 @@ transposable_kernel(const T* __restrict__ dense, int64_t ld, int64_t nmajor4, in
 template <typename T, bool ABS, bool TRANS>
 int launch(const void* dense, int64_t ld, int64_t m, int64_t k, void* sparse, uint8_t* mask, hipStream_t s) {
   const int64_t nmajor4 = (TRANS ? k : m) / 4, nminor8 = (TRANS ? m : k) / 8;     // both extents are multiples of 32
-  dim3 grid((unsigned)nmajor4, (unsigned)((nminor8 + kThreads - 1) / kThreads));
+  dim3 grid((unsigned)(nmajor4 * ((nminor8 + kThreads - 1) / kThreads)));
   hipLaunchKernelGGL((transposable_kernel<T, ABS, TRANS>), grid, dim3(kThreads), 0, s, (const T*)dense, ld, nmajor4, nminor8,
                      (T*)sparse, mask);
   return check_launch("tf24_transposable_mask");
