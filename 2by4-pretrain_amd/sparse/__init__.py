@@ -12,6 +12,7 @@ from .dense_ops import (soft_threshold24, sparse24, MVUE24_approx,
                         soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton)
 from .sparse_linear_transpose import SparseLinearTranspose, sparse_linear_transpose
 from .sparse_semi_structured_linear import sparse_semi_structured_linear
+from .GELUglu import GELUglu, gelu_glu
 from .sparse_ops import MyLinear, SparseLinear, SoftThreshold, SoftThresholdLinear, Sparse24
 
 __all__ = [
@@ -22,5 +23,6 @@ __all__ = [
     "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
     "SparseLinearTranspose", "sparse_linear_transpose",
     "sparse_semi_structured_linear",
+    "GELUglu", "gelu_glu",
     "MyLinear", "SparseLinear", "SoftThreshold", "SoftThresholdLinear", "Sparse24",
 ]

@@ -225,6 +225,27 @@ int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype,
 int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense);
 
 /*
+ * GELU-GLU: the last dimension of `in` [rows, cols] holds [x | gate] (cols/2 each);
+ *     out[r, c] = x[r, c] * 0.5 * gate * (1 + tanh(sqrt(2/pi) * (gate + 0.044715 * gate^3))),  c < cols/2
+ * and its backward pass
+ *     grad_in[r, c]          = grad_out[r, c] * gelu_tanh(gate)
+ *     grad_in[r, cols/2 + c] = grad_out[r, c] * x * d gelu_tanh(gate) / d gate.
+ * Replaces the Triton kernels of sparse/GELUglu.py (forward :16-47 and :51-80, backward :83-153;
+ * launchers :156-236).  Arithmetic is float32 with one rounding to `dtype` (F32|F16|BF16); the
+ * reference computes in the storage type.
+ *   layout  TF24_ROW_MAJOR: element (r, c) at r*ld + c (the reference's stride[-1] == 1 path);
+ *           TF24_COL_MAJOR: at c*ld + r (its "fall back to 2D" path for transposed storage).
+ *           `out` / `grad_out` are [rows, cols/2], `grad_in` is [rows, cols], in the same layout.
+ * cols must be even.  16-byte accesses are used when the extents, leading dimensions and pointers
+ * allow (multiples of 8 elements, 16-byte aligned); any other shape runs element-wise.
+ */
+int tf24_gelu_glu_forward(const void* in, int dtype, int layout, int64_t ld_in, int64_t rows, int64_t cols,
+                          void* out, int64_t ld_out, void* stream);
+int tf24_gelu_glu_backward(const void* grad_out, int64_t ld_grad_out, const void* in, int dtype, int layout,
+                           int64_t ld_in, int64_t rows, int64_t cols, void* grad_in, int64_t ld_grad_in,
+                           void* stream);
+
+/*
  * out[c, r] = in[r, c] for 2-byte (F16|BF16) and 1-byte (E4M3|E5M2|U8) elements; in [rows, cols] with
  * leading dimension ld_in, out [cols, rows] with ld_out.  No counterpart in the reference (CUTLASS
  * reads either operand layout): it feeds tf24_spmm's fast kernel, which wants an 8-bit dense operand

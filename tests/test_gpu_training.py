@@ -262,3 +262,41 @@ def test_masked_decay_adamw_kernel(cuda, gdt):
         ref_opt.step()
         assert torch.allclose(par.detach(), ref_par.detach(), rtol=1e-5, atol=1e-7)
         assert torch.allclose(plain.detach(), ref_plain.detach(), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.float16, 1e-3), (torch.bfloat16, 8e-3)])
+@pytest.mark.parametrize("shape", [(4, 32, 256), (3, 5, 24), (2, 7, 10), (1, 1, 2)])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_gelu_glu_forward_backward(cuda, dtype, tol, shape, transposed):
+    """GELUglu against the float64 oracle.  Tolerances: float32 arithmetic then one rounding to the
+    storage type, so 2e-6 (float32), 2^-10 (float16) and 2^-7 (bfloat16) of the largest
+    magnitude; `transposed` stores the last dimension strided (the reference's 2-d path)."""
+    import sparse
+    g = torch.Generator().manual_seed(41)
+    a, b, c = shape
+    inp = (2 * torch.randn(a * b, c, generator=g)).to(dtype)
+    go = torch.randn(a * b, c // 2, generator=g).to(dtype)
+    dev_in = inp.to(cuda)
+    if transposed:
+        dev_in = dev_in.t().contiguous().t()                    # same values, column-major storage
+    dev_in = dev_in.view(a, b, c).requires_grad_(True)
+    out = sparse.GELUglu()(dev_in)
+    want = oracle.gelu_glu_forward(inp.view(a, b, c))
+    assert out.shape == (a, b, c // 2) and out.dtype == dtype
+    scale = want.abs().max().item()
+    assert (out.double().cpu() - want).abs().max().item() <= tol * scale + 1e-30
+    out.backward(go.to(cuda).view(a, b, c // 2))
+    want_g = oracle.gelu_glu_backward(go.view(a, b, c // 2), inp.view(a, b, c))
+    assert dev_in.grad.shape == (a, b, c) and dev_in.grad.dtype == dtype
+    gscale = want_g.abs().max().item()
+    assert (dev_in.grad.double().cpu() - want_g).abs().max().item() <= tol * gscale + 1e-30
+
+
+def test_gelu_glu_errors(cuda):
+    import sparse
+    with pytest.raises(RuntimeError):
+        sparse.gelu_glu.apply(torch.zeros(2, 3, 5, device=cuda))          # odd last dimension
+    with pytest.raises(RuntimeError):
+        sparse.gelu_glu.apply(torch.zeros(2, 3, 4))                       # not on the GPU
+    with pytest.raises(AssertionError):
+        sparse.gelu_glu.apply(torch.zeros(6, 4, device=cuda))             # the reference asserts a 3-d input

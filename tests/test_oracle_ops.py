@@ -220,3 +220,24 @@ def test_adamw_oracle_matches_torch_adamw_and_closed_form():
     b = oracle.adamw_masked_decay(p, oracle.masked_add(grad, p, mask, 2e-4), m, v, None, 6, **hyp)
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+
+
+def test_gelu_glu_oracle_matches_torch_gelu_and_autograd():
+    """The GELU-GLU oracle is pinned by torch's own tanh-GELU and by autograd's gradient of
+    gelu(gate) * x: swapped halves, a dropped factor or a sign error fails one of them."""
+    g = torch.Generator().manual_seed(31)
+    inp = (3 * torch.randn(5, 7, 24, generator=g, dtype=torch.float64)).requires_grad_(True)
+    go = torch.randn(5, 7, 12, generator=g, dtype=torch.float64)
+    out = oracle.gelu_glu_forward(inp.detach())
+    x, gate = inp[..., :12], inp[..., 12:]
+    ref = torch.nn.functional.gelu(gate, approximate='tanh') * x
+    assert torch.allclose(out, ref.detach(), rtol=1e-12, atol=1e-14)
+    (want,) = torch.autograd.grad(ref, inp, go)
+    got = oracle.gelu_glu_backward(go, inp.detach())
+    assert got.shape == inp.shape and torch.allclose(got, want, rtol=1e-10, atol=1e-12)
+    # special values: gate = 0 gives out = 0 and d/dgate = x/2; a large gate passes x through
+    z = torch.tensor([[[2.0, -3.0, 0.0, 0.0]]], dtype=torch.float64)
+    assert oracle.gelu_glu_forward(z).abs().max() == 0
+    assert torch.allclose(oracle.gelu_glu_backward(torch.ones(1, 1, 2, dtype=torch.float64), z)[..., 2:], torch.tensor([1.0, -1.5], dtype=torch.float64))
+    big = torch.tensor([[[2.0, -3.0, 30.0, -30.0]]], dtype=torch.float64)
+    assert torch.allclose(oracle.gelu_glu_forward(big), torch.tensor([[[60.0, 0.0]]], dtype=torch.float64), atol=1e-9)
