@@ -54,17 +54,27 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
                                             int has_mask, int mask_dtype, int64_t mask_ld, int has_rand, int64_t rand_ld,
                                             int out_dtype) {
   const char* fn = "tf24_prune_compress";
-  if (!is_float_dtype(in_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
-  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && !is_float8(out_dtype))
+  if (!is_float_dtype(in_dtype) && in_dtype != TF24_I8) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
+  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && !is_8bit(out_dtype))
     return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
+  if ((in_dtype == TF24_I8) != (out_dtype == TF24_I8))
+    return fail(TF24_ERR_DTYPE, "%s: int8 values come from an int8 dense matrix only (input dtype %d, output dtype %d)", fn, in_dtype, out_dtype);
+  if (in_dtype == TF24_I8 && (mode == TF24_PRUNE_MVUE || mode == TF24_PRUNE_MVUE_PACKED))
+    return fail(TF24_ERR_ARG, "%s: MVUE24 rescales the kept values and is not defined for int8", fn);
   if (!is_layout(layout)) return fail(TF24_ERR_ARG, "%s: bad layout %d", fn, layout);
-  const int64_t min_rows = 32, min_cols = is_float8(out_dtype) ? 128 : 64;
+  const int64_t min_rows = 32, min_cols = is_8bit(out_dtype) ? 128 : 64;
   if (m < min_rows || m % min_rows || k < min_cols || k % min_cols)
     return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld) is not supported: both dimensions must be >= and a multiple of (%lld, %lld)",
                 fn, (long long)m, (long long)k, (long long)min_rows, (long long)min_cols);
   if (m * (k / 8) > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "%s: matrix too large (%lld x %lld)", fn, (long long)m, (long long)k);
   int rc = check_ld(fn, "dense", layout, ld, m, k);
   if (rc) return rc;
+  if (in_dtype == TF24_I8) {
+    if (has_mask && mask_dtype != TF24_U8) return fail(TF24_ERR_DTYPE, "%s: int8 input takes a byte mask (dtype %d given)", fn, mask_dtype);
+    // column-major int8: a lane reads 16 rows of a column with one 16-byte load
+    if (layout == TF24_COL_MAJOR && (ld % 16 || (has_mask && mask_ld % 16)))
+      return fail(TF24_ERR_STRIDE, "%s: column-major int8 input needs leading dimensions that are multiples of 16", fn);
+  }
   switch (mode) {
     case TF24_PRUNE_MAGNITUDE:
       break;
@@ -91,13 +101,15 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
 extern "C" int tf24_prune_compress_dual_validate(int in_dtype, int64_t ld, int64_t m, int64_t k, int mask_dtype,
                                                  int64_t mask_ld, int out_dtype, int out_layout) {
   const char* fn = "tf24_prune_compress_dual";
-  if (!is_float_dtype(in_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
-  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && !is_float8(out_dtype))
+  if (!is_float_dtype(in_dtype) && in_dtype != TF24_I8) return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
+  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && !is_8bit(out_dtype))
     return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
+  if ((in_dtype == TF24_I8) != (out_dtype == TF24_I8))
+    return fail(TF24_ERR_DTYPE, "%s: int8 values come from an int8 dense matrix only (input dtype %d, output dtype %d)", fn, in_dtype, out_dtype);
   if (!is_mask_dtype(mask_dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported mask dtype %d", fn, mask_dtype);
   if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
     return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, out_layout);
-  const int64_t unit = is_float8(out_dtype) ? 128 : 64;
+  const int64_t unit = is_8bit(out_dtype) ? 128 : 64;
   if (m < unit || m % unit || k < unit || k % unit)
     return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld) is not supported: both dimensions must be >= and a multiple of %lld",
                 fn, (long long)m, (long long)k, (long long)unit);

@@ -71,8 +71,8 @@ extern "C" int tf24_repack(const void* values_in, const void* meta_in, int dtype
                            void* values_out, void* meta_out, void* stream) {
   using namespace tf24;
   const char* fn = "tf24_repack";
-  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_float8(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
-  const int64_t kp = is_float8(dtype) ? 128 : 64;
+  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_8bit(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
+  const int64_t kp = is_8bit(dtype) ? 128 : 64;
   if (m <= 0 || k <= 0 || k % kp) return fail(TF24_ERR_SHAPE, "%s: k=%lld must be a positive multiple of %lld", fn, (long long)k, (long long)kp);
   if (from_layout != TF24_COMPRESSED_CANONICAL && from_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, from_layout);
   if (!values_in || !meta_in || !values_out || !meta_out) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
@@ -89,18 +89,19 @@ extern "C" int tf24_repack(const void* values_in, const void* meta_in, int dtype
 extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, int layout, int64_t m, int64_t k,
                                void* dense_out, void* stream) {
   using namespace tf24;
-  const int64_t mult = is_float8(dtype) ? 32 : 16;
+  const int64_t mult = is_8bit(dtype) ? 32 : 16;
   if (m <= 0 || k <= 0 || k % mult) return fail(TF24_ERR_SHAPE, "tf24_decompress: k=%lld must be a positive multiple of %lld", (long long)k, (long long)mult);
   if (!values || !meta || !dense_out) return fail(TF24_ERR_ARG, "tf24_decompress: null pointer");
   if (layout != TF24_COMPRESSED_CANONICAL && layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_decompress: bad compressed layout %d", layout);
   const bool panel = layout == TF24_COMPRESSED_PANEL;
-  if (panel && k % (is_float8(dtype) ? 128 : 64)) return fail(TF24_ERR_SHAPE, "tf24_decompress: panel layout needs whole panels (k=%lld)", (long long)k);
+  if (panel && k % (is_8bit(dtype) ? 128 : 64)) return fail(TF24_ERR_SHAPE, "tf24_decompress: panel layout needs whole panels (k=%lld)", (long long)k);
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case TF24_F16: return launch<f16_t>(values, meta, panel, m, k, dense_out, s);
     case TF24_BF16: return launch<bf16_t>(values, meta, panel, m, k, dense_out, s);
     case TF24_E4M3: return launch<e4m3_t>(values, meta, panel, m, k, dense_out, s);
     case TF24_E5M2: return launch<e5m2_t>(values, meta, panel, m, k, dense_out, s);
+    case TF24_I8: return launch<i8_t>(values, meta, panel, m, k, dense_out, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_decompress: unsupported dtype %d", dtype);
 }

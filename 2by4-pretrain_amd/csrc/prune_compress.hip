@@ -7,6 +7,8 @@
 // live entirely in its registers), a 256-lane block covers 8R rows x 128 columns, and the
 // compressed tile is transposed through LDS so that values and metadata leave row-major with
 // full-line stores.
+#include <type_traits>
+
 #include "tf24_common.hpp"
 
 namespace tf24 {
@@ -267,6 +269,10 @@ int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t 
                   int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
   if constexpr (MODE != TF24_PRUNE_MASK) {
     return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, rand_packed, values, meta, panel, s);
+  } else if constexpr (std::is_same<In, i8_t>::value) {
+    // int8 matrices take byte masks only (the column kernel reads 16 rows per lane: 16-byte mask loads)
+    if (mask_dtype != TF24_U8) return fail(TF24_ERR_DTYPE, "tf24_prune_compress: int8 input takes a byte mask (dtype %d given)", mask_dtype);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
   } else {
     switch (mask_dtype) {
       case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
@@ -288,7 +294,8 @@ int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m
       return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
     case TF24_PRUNE_MVUE:
     case TF24_PRUNE_MVUE_PACKED:
-      return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      if constexpr (std::is_same<Out, i8_t>::value) break;        // refused by the validator
+      else return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
   }
   return fail(TF24_ERR_ARG, "tf24_prune_compress: bad mode %d", mode);
 }
@@ -326,6 +333,7 @@ extern "C" int tf24_prune_compress(const void* dense, int in_dtype, int layout, 
     case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
     case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
     case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_I8: return dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported input dtype %d", in_dtype);
 }

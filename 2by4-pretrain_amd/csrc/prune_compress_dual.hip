@@ -190,6 +190,7 @@ extern "C" int tf24_prune_compress_dual(const void* dense, int in_dtype, int64_t
     case TF24_F32: return dispatch_out<float>(out_dtype, mask_dtype, dense, ld, m, k, mask, mask_ld, values, meta, values_t, meta_t, panel, s);
     case TF24_F16: return dispatch_out<f16_t>(out_dtype, mask_dtype, dense, ld, m, k, mask, mask_ld, values, meta, values_t, meta_t, panel, s);
     case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mask_dtype, dense, ld, m, k, mask, mask_ld, values, meta, values_t, meta_t, panel, s);
+    case TF24_I8: return dispatch_mask<i8_t, i8_t>(mask_dtype, dense, ld, m, k, mask, mask_ld, values, meta, values_t, meta_t, panel, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress_dual: unsupported input dtype %d", in_dtype);
 }

@@ -28,12 +28,14 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int8v __attribute__((ext_vector_type(8)));
+typedef int int16v __attribute__((ext_vector_type(16)));
 
 // ---- element traits: KSTEP = dense depth of one 16x16 instruction; all types move 64 bytes of
 // compressed A and 128 bytes of B per row per step.
 template <typename T> struct mma16;
 template <> struct mma16<f16_t> {
   static constexpr int KSTEP = 64;
+  using acc_t = float4v;
   template <int ABID>
   static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_16x16x64_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half16, b), c, idx, 0, ABID);
@@ -41,6 +43,7 @@ template <> struct mma16<f16_t> {
 };
 template <> struct mma16<bf16_t> {
   static constexpr int KSTEP = 64;
+  using acc_t = float4v;
   template <int ABID>
   static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_16x16x64_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x16, b), c, idx, 0, ABID);
@@ -48,6 +51,7 @@ template <> struct mma16<bf16_t> {
 };
 template <> struct mma16<e4m3_t> {
   static constexpr int KSTEP = 128;
+  using acc_t = float4v;
   template <int ABID>
   static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_16x16x128_fp8_fp8(a, b, c, idx, 0, 0);
@@ -55,9 +59,19 @@ template <> struct mma16<e4m3_t> {
 };
 template <> struct mma16<e5m2_t> {
   static constexpr int KSTEP = 128;
+  using acc_t = float4v;
   template <int ABID>
   static __device__ __forceinline__ float4v run(int4v a, int8v b, float4v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_16x16x128_bf8_bf8(a, b, c, idx, 0, 0);
+  }
+};
+
+template <> struct mma16<i8_t> {
+  static constexpr int KSTEP = 128;
+  using acc_t = int4v;
+  template <int ABID>
+  static __device__ __forceinline__ int4v run(int4v a, int8v b, int4v c, int idx) {
+    return __builtin_amdgcn_smfmac_i32_16x16x128_i8(a, b, c, idx, 0, 0);
   }
 };
 
@@ -66,6 +80,23 @@ __device__ __forceinline__ float apply_act(float v, int act) {
   if (act == TF24_ACT_SILU) return v / (1.0f + __expf(-v));
   if (act == TF24_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
   return v;
+}
+
+// An accumulator element -> the finished output element.  Floating accumulators: scale, bias,
+// activation, one rounding.  Integer accumulators (int8 operands): bias and ReLU in int32, exact.
+template <typename OutT> __device__ __forceinline__ OutT to_out(float v) { return from_float<OutT>(v); }
+template <typename OutT> __device__ __forceinline__ OutT to_out(int v) { return (OutT)v; }
+template <typename OutT>
+__device__ __forceinline__ float finish_value(float accv, float scale, const OutT* bias, int64_t row, int act) {
+  float v = accv * scale;
+  if (bias) v += to_float(bias[row]);
+  return apply_act(v, act);
+}
+template <typename OutT>
+__device__ __forceinline__ int finish_value(int accv, float, const OutT* bias, int64_t row, int act) {
+  int v = accv;
+  if (bias) v += (int)bias[row];
+  return (act == TF24_ACT_RELU && v < 0) ? 0 : v;
 }
 
 // The output pass of the tiled kernel is compiled three times: without bias and activation, with a
@@ -78,6 +109,14 @@ __device__ __forceinline__ float finish_element(float accv, float scale, const O
   float v = accv * scale;
   if constexpr (MODE == EPI_BIAS) { if (row_ok) v += to_float(bias[row]); }
   if constexpr (MODE == EPI_RUNTIME) { if (bias && row_ok) v += to_float(bias[row]); v = apply_act(v, act); }
+  return v;
+}
+
+template <int MODE, typename OutT>
+__device__ __forceinline__ int finish_element(int accv, float, const OutT* bias, int64_t row, bool row_ok, int act) {
+  int v = accv;
+  if constexpr (MODE != EPI_PLAIN) { if (bias && row_ok) v += (int)bias[row]; }
+  if constexpr (MODE == EPI_RUNTIME) { if (act == TF24_ACT_RELU && v < 0) v = 0; }
   return v;
 }
 
@@ -99,11 +138,13 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
   const int li = lane & 15, lk = lane >> 4;
   const int64_t a_pitch = (k / 2) * ES;               // bytes per row of compressed values
   const int64_t m_pitch = k / 8;                      // bytes per row of metadata
-  float4v acc[2][2];
+  typename mma16<T>::acc_t acc[2][2];
 #pragma unroll
   for (int ti = 0; ti < 2; ti++)
 #pragma unroll
-    for (int tj = 0; tj < 2; tj++) acc[ti][tj] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int tj = 0; tj < 2; tj++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[ti][tj][r] = 0;
 
   for (int64_t k0 = 0; k0 < k; k0 += KSTEP) {
     int4v af[2];
@@ -154,11 +195,7 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
       const int64_t row = i0 + ti * 16 + lk * 4;
       OutT o[4];
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        float v = acc[ti][tj][r] * scale;
-        if (bias) v += to_float(bias[row + r]);
-        o[r] = from_float<OutT>(apply_act(v, act));
-      }
+      for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_value(acc[ti][tj][r], scale, bias, row + r, act));
       if constexpr (C_JMAJOR) {
         *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
       } else {
@@ -193,23 +230,39 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 // ------------------------------------------------------------------------------------------
 template <typename T> struct mma32;
 template <> struct mma32<f16_t> {
+  using acc_t = float16v;
+  using acc4_t = float4v;
   static __device__ __forceinline__ float16v run(int4v a, int8v b, float16v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_32x32x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half16, b), c, idx, 0, 0);
   }
 };
 template <> struct mma32<bf16_t> {
+  using acc_t = float16v;
+  using acc4_t = float4v;
   static __device__ __forceinline__ float16v run(int4v a, int8v b, float16v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_32x32x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x16, b), c, idx, 0, 0);
   }
 };
 template <> struct mma32<e4m3_t> {
+  using acc_t = float16v;
+  using acc4_t = float4v;
   static __device__ __forceinline__ float16v run(int4v a, int8v b, float16v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(a, b, c, idx, 0, 0);
   }
 };
 template <> struct mma32<e5m2_t> {
+  using acc_t = float16v;
+  using acc4_t = float4v;
   static __device__ __forceinline__ float16v run(int4v a, int8v b, float16v c, int idx) {
     return __builtin_amdgcn_smfmac_f32_32x32x64_bf8_bf8(a, b, c, idx, 0, 0);
+  }
+};
+
+template <> struct mma32<i8_t> {
+  using acc_t = int16v;
+  using acc4_t = int4v;
+  static __device__ __forceinline__ int16v run(int4v a, int8v b, int16v c, int idx) {
+    return __builtin_amdgcn_smfmac_i32_32x32x64_i8(a, b, c, idx, 0, 0);
   }
 };
 
@@ -354,13 +407,13 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     for (int q = 0; q < NCOPY; q++) issue_one(q, st, dst);
   };
 
-  float16v acc[C::TI][C::TJ];
+  typename mma32<T>::acc_t acc[C::TI][C::TJ];
 #pragma unroll
   for (int ti = 0; ti < C::TI; ti++)
 #pragma unroll
     for (int tj = 0; tj < C::TJ; tj++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[ti][tj][r] = 0.0f;
+      for (int r = 0; r < 16; r++) acc[ti][tj][r] = 0;
 
   // ---- fragment offsets (swizzled)
   const int a_row = wi * C::WI + l32, b_row = wj * C::WJ + l32;
@@ -506,7 +559,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   }
   mma_step(1, 0, false, 0, 0, false, 0, 0);       // the last step
 
-  // ---- split-K: park the float32 accumulators in the workspace, in register order (every group of
+  // ---- split-K: park the 32-bit accumulators in the workspace, in register order (every group of
   // four accumulators is one contiguous 16-byte-per-lane slab); spmm_reduce_splits finishes the job.
   if (splits > 1) {
     float* base = partial + (int64_t)unit * (C::BI * C::BJ);
@@ -517,8 +570,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 #pragma unroll
         for (int g = 0; g < 4; g++) {
           const int slab = (ti * C::TJ + tj) * 4 + g;
-          float4v v = {acc[ti][tj][g * 4], acc[ti][tj][g * 4 + 1], acc[ti][tj][g * 4 + 2], acc[ti][tj][g * 4 + 3]};
-          *reinterpret_cast<float4v*>(base + ((int64_t)slab * C::THREADS + tid) * 4) = v;
+          typename mma32<T>::acc4_t v = {acc[ti][tj][g * 4], acc[ti][tj][g * 4 + 1], acc[ti][tj][g * 4 + 2], acc[ti][tj][g * 4 + 3]};
+          *reinterpret_cast<typename mma32<T>::acc4_t*>(base + ((int64_t)slab * C::THREADS + tid) * 4) = v;
         }
     return;
   }
@@ -551,7 +604,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
               OutT o[4];
   #pragma unroll
               for (int r = 0; r < 4; r++) {
-                o[r] = from_float<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
+                o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
               }
               const int ch = ti * 4 + g;
               *reinterpret_cast<Pack<OutT, 4>*>(stage + jl * 256 + ((ch ^ (jl & 15)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
@@ -587,7 +640,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
                 const int il = ti * 32 + g * 8 + lh * 4 + r;
                 const int64_t row = i0 + wi * C::WI + il;
                 *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ ((il >> 1) & 7)) * 16) + (jl & 7) * 2) =
-                    from_float<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row, row < n_sparse, act));
+                    to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row, row < n_sparse, act));
               }
           }
         const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
@@ -612,7 +665,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             OutT o[4];
   #pragma unroll
             for (int r = 0; r < 4; r++) {
-              o[r] = from_float<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, true, act));
+              o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, true, act));
             }
             if constexpr (C_JMAJOR) {
               *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
@@ -630,9 +683,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 }
 
 // Second pass of a split-K product: a block handles one eighth of a tile (the accumulator groups
-// `slab` of one ti), same lane -> element mapping as spmm_pipe; sums the `splits` float32 partial
-// tiles and applies scale / bias / activation / conversion.
-template <typename OutT, bool C_JMAJOR, typename C>
+// `slab` of one ti), same lane -> element mapping as spmm_pipe; sums the `splits` partial tiles
+// (float32, or int32 for int8 operands) and applies scale / bias / activation / conversion.
+template <typename Acc4, typename OutT, bool C_JMAJOR, typename C>
 __global__ void __launch_bounds__(C::THREADS)
 spmm_reduce_splits(const float* __restrict__ partial, int splits, int tiles_i, int tiles_j, int64_t n_sparse, int64_t n_dense,
                    OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
@@ -650,21 +703,17 @@ spmm_reduce_splits(const float* __restrict__ partial, int splits, int tiles_i, i
   // gridDim.y blocks share the NSLAB accumulator groups of the tile
   for (int slab = blockIdx.y; slab < NSLAB; slab += gridDim.y) {
     const int ti = slab / (C::TJ * 4), tj = (slab / 4) % C::TJ, g = slab % 4;
-    float4v sum = {0.f, 0.f, 0.f, 0.f};
+    Acc4 sum = {0, 0, 0, 0};
     for (int sp = 0; sp < splits; sp++) {
       const float* base = partial + ((int64_t)sp * ntiles + tile) * (C::BI * C::BJ);
-      sum += *reinterpret_cast<const float4v*>(base + ((int64_t)slab * C::THREADS + tid) * 4);
+      sum += *reinterpret_cast<const Acc4*>(base + ((int64_t)slab * C::THREADS + tid) * 4);
     }
     const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
     const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
     if (col >= n_dense || row >= n_sparse) continue;
     OutT o[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      float v = sum[r] * scale;
-      if (bias) v += to_float(bias[row + r]);
-      o[r] = from_float<OutT>(apply_act(v, act));
-    }
+    for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_value(sum[r], scale, bias, row + r, act));
     if constexpr (C_JMAJOR) {
       *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
     } else {
@@ -716,10 +765,10 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   if (splits > 1) {
     dim3 rgrid((unsigned)(tiles_i * tiles_j), 8);
     if (jm)
-      hipLaunchKernelGGL((spmm_reduce_splits<OutT, true, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
+      hipLaunchKernelGGL((spmm_reduce_splits<typename mma32<T>::acc4_t, OutT, true, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
                          n_sparse, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
     else
-      hipLaunchKernelGGL((spmm_reduce_splits<OutT, false, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
+      hipLaunchKernelGGL((spmm_reduce_splits<typename mma32<T>::acc4_t, OutT, false, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
                          n_sparse, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
   }
   return check_launch("tf24_spmm");
@@ -746,7 +795,12 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  void* workspace, int64_t workspace_bytes, hipStream_t s) {
   // the tiled kernel reads a k-strided dense operand through transposing LDS reads (16-bit types only)
-  if (panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64 && n_dense >= 64) {
+  const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64 && n_dense >= 64;
+  if constexpr (std::is_same<T, i8_t>::value) {        // integer product: int32 accumulators, results and bias
+    if (tiled) return launch_tiled<T, int32_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+    return launch_general<T, int32_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+  } else {
+  if (tiled) {
     switch (out_dtype) {
       case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
       case TF24_BF16: return launch_tiled<T, bf16_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
@@ -759,6 +813,7 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
     case TF24_F32: return launch_general<T, float>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_spmm: unsupported output dtype %d", out_dtype);
+  }
 }
 
 }  // namespace
@@ -768,9 +823,15 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
                                   int out_dtype, int c_layout, int64_t ldc, int activation) {
   using namespace tf24;
   const char* fn = "tf24_spmm";
-  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_float8(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported operand dtype %d", fn, dtype);
-  if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && out_dtype != TF24_F32) return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
-  const bool eight = is_float8(dtype);
+  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_8bit(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported operand dtype %d", fn, dtype);
+  if (dtype == TF24_I8) {
+    // integer product (.cu:594-637): int32 results, no or ReLU activation
+    if (out_dtype != TF24_I32) return fail(TF24_ERR_DTYPE, "%s: int8 operands give int32 results (output dtype %d)", fn, out_dtype);
+    if (activation != TF24_ACT_NONE && activation != TF24_ACT_RELU) return fail(TF24_ERR_ARG, "%s: int8 operands support no activation or ReLU (%d)", fn, activation);
+  } else if (out_dtype != TF24_F16 && out_dtype != TF24_BF16 && out_dtype != TF24_F32) {
+    return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
+  }
+  const bool eight = is_8bit(dtype);
   const int64_t kmult = eight ? 128 : 64, dmult = eight ? 16 : 8;
   if (n_sparse <= 0 || n_sparse % 32) return fail(TF24_ERR_SHAPE, "%s: sparse operand rows %lld must be a positive multiple of 32", fn, (long long)n_sparse);
   if (k <= 0 || k % kmult) return fail(TF24_ERR_SHAPE, "%s: inner dimension %lld must be a positive multiple of %lld", fn, (long long)k, (long long)kmult);
@@ -789,7 +850,7 @@ extern "C" int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_
   using namespace tf24;
   const int64_t big = (int64_t)1 << 40;
   int splits;
-  if (is_float8(dtype)) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
+  if (is_8bit(dtype)) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
   else splits = choose_splits<f16_t, TiledCfg>(n_sparse, k, n_dense, big);
   if (splits < 2) return 0;
   const int64_t tiles = ((n_sparse + TiledCfg::BI - 1) / TiledCfg::BI) * ((n_dense + TiledCfg::BJ - 1) / TiledCfg::BJ);
@@ -807,7 +868,9 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout,
   if (a_layout != TF24_COMPRESSED_CANONICAL && a_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_spmm: bad compressed layout %d", a_layout);
   const bool panel = a_layout == TF24_COMPRESSED_PANEL;
   hipStream_t s = (hipStream_t)stream;
+  if (dtype == TF24_I8 && scale != 1.0f) return fail(TF24_ERR_ARG, "tf24_spmm: int8 products are exact, scale must be 1 (%g given)", (double)scale);
   switch (dtype) {
+    case TF24_I8: return dispatch_out<i8_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
     case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
     case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
     case TF24_E5M2: return dispatch_out<e5m2_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);

@@ -17,6 +17,7 @@ struct f16_t { uint16_t bits; };
 struct bf16_t { uint16_t bits; };
 struct e4m3_t { uint8_t bits; };
 struct e5m2_t { uint8_t bits; };
+struct i8_t { uint8_t bits; };      // two's-complement int8
 
 template <typename T> struct dtype_of;
 template <> struct dtype_of<float> { static constexpr int value = TF24_F32; };
@@ -24,11 +25,15 @@ template <> struct dtype_of<f16_t> { static constexpr int value = TF24_F16; };
 template <> struct dtype_of<bf16_t> { static constexpr int value = TF24_BF16; };
 template <> struct dtype_of<e4m3_t> { static constexpr int value = TF24_E4M3; };
 template <> struct dtype_of<e5m2_t> { static constexpr int value = TF24_E5M2; };
+template <> struct dtype_of<i8_t> { static constexpr int value = TF24_I8; };
+template <> struct dtype_of<int32_t> { static constexpr int value = TF24_I32; };
 __host__ __device__ inline bool is_float8(int dt) { return dt == TF24_E4M3 || dt == TF24_E5M2; }
+// value types stored one byte per element: 128 dense columns per panel, int32 metadata words
+__host__ __device__ inline bool is_8bit(int dt) { return is_float8(dt) || dt == TF24_I8; }
 template <> struct dtype_of<uint8_t> { static constexpr int value = TF24_U8; };
 
 __host__ __device__ inline int dtype_size(int dt) {
-  return dt == TF24_F32 ? 4 : (dt == TF24_F16 || dt == TF24_BF16) ? 2 : 1;
+  return (dt == TF24_F32 || dt == TF24_I32) ? 4 : (dt == TF24_F16 || dt == TF24_BF16) ? 2 : 1;
 }
 
 // ---------------------------------------------------------------- conversions to float (exact)
@@ -107,6 +112,12 @@ __host__ __device__ inline uint8_t float_to_e5m2(float f) {
   return (uint8_t)(r | sign);
 }
 template <> __device__ __forceinline__ e5m2_t from_float<e5m2_t>(float f) { return e5m2_t{float_to_e5m2(f)}; }
+// int8: exact for the integers an int8 dense operand holds (the only input the int8 path accepts)
+template <> __device__ __forceinline__ i8_t from_float<i8_t>(float f) {
+  const float c = f < -128.0f ? -128.0f : (f > 127.0f ? 127.0f : f);
+  return i8_t{(uint8_t)(int8_t)(int)c};
+}
+__device__ __forceinline__ float to_float(i8_t v) { return (float)(int8_t)v.bits; }
 __device__ __forceinline__ float to_float(e5m2_t v) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)((uint16_t)v.bits << 8));
 }

@@ -54,7 +54,7 @@ extern "C" int tf24_transpose(const void* in, int dtype, int64_t ld_in, int64_t 
   using namespace tf24;
   const int es = dtype_size(dtype);
   const int64_t v = 16 / es;
-  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_float8(dtype) && dtype != TF24_U8)
+  if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_8bit(dtype) && dtype != TF24_U8)
     return fail(TF24_ERR_DTYPE, "tf24_transpose: unsupported dtype %d", dtype);
   if (rows <= 0 || cols <= 0 || rows % v || cols % v)
     return fail(TF24_ERR_SHAPE, "tf24_transpose: rows and cols must be positive multiples of %lld", (long long)v);

@@ -12,7 +12,7 @@ _LIB_NAME = "lib2by4_gfx950.so"
 _lib = None
 
 # enums of tf24.h
-F32, F16, BF16, E4M3, U8, E5M2 = 0, 1, 2, 3, 4, 5
+F32, F16, BF16, E4M3, U8, E5M2, I8, I32 = 0, 1, 2, 3, 4, 5, 6, 7
 ROW_MAJOR, COL_MAJOR = 0, 1
 PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE, PRUNE_MVUE_PACKED = 0, 1, 2, 3
 ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
@@ -85,6 +85,16 @@ def dtype_code(dtype):
         return _DTYPES[dtype]
     except KeyError:
         raise RuntimeError(f"dtype {dtype} is not supported by the gfx950 2:4 library") from None
+
+
+def operand_code(dtype):
+    """dtype code of a matrix of values: like dtype_code, except that int8 / int32 are the integer
+    value types (dtype_code reads int8 as a byte mask)."""
+    if dtype == torch.int8:
+        return I8
+    if dtype == torch.int32:
+        return I32
+    return dtype_code(dtype)
 
 
 def check(rc):

@@ -30,16 +30,18 @@ _Config = namedtuple("_SEMI_STRUCTURED_SPARSE_CONFIG",
 _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG = {
     torch.float8_e4m3fn: _Config(10, 32, 128, 16, 16),
     torch.float8_e5m2: _Config(10, 32, 128, 16, 16),
+    torch.int8: _Config(10, 32, 128, 16, 16),
     torch.float16: _Config(9, 32, 64, 8, 8),
     torch.bfloat16: _Config(9, 32, 64, 8, 8),
 }
 
 
 _FLOAT8 = (torch.float8_e4m3fn, torch.float8_e5m2)
+_EIGHT_BIT = _FLOAT8 + (torch.int8,)          # 128 dense columns per panel, int32 metadata words
 
 
 def _indices_dtype(values_dtype):
-    if values_dtype in _FLOAT8:
+    if values_dtype in _EIGHT_BIT:
         return torch.int32
     if values_dtype in (torch.float16, torch.bfloat16):
         return torch.int16
@@ -68,8 +70,17 @@ def _compress(original, dtype, MVUE24, mask, rand, panel):
     values = buf[: m * n // 2]
     meta = buf[m * n // 2:].view(_indices_dtype(dtype))
 
+    if (dtype == torch.int8) != (original.dtype == torch.int8):
+        raise RuntimeError(f"int8 values are taken from an int8 dense tensor only (tensor {original.dtype}, dtype {dtype})")
+    if dtype == torch.int8 and MVUE24:
+        raise RuntimeError("MVUE24 rescales the kept values and is not defined for int8")
     dense = N.as_matrix(original)
     layout, ld = N.layout_of(dense)
+    if dtype == torch.int8 and layout == N.COL_MAJOR and ld % 16:
+        dense = dense.contiguous()                   # column-major int8 is read 16 rows at a time
+        layout, ld = N.layout_of(dense)
+    if dtype == torch.int8 and mask is not None and mask.dtype not in (torch.bool, torch.uint8):
+        mask = mask != 0                             # int8 matrices take byte masks
     mode, mask_t, rand_t = N.PRUNE_MAGNITUDE, None, None
     mask_ld = rand_ld = 0
     mask_code = N.U8
@@ -96,9 +107,9 @@ def _compress(original, dtype, MVUE24, mask, rand, panel):
         rand_t = N.as_matrix(rand.float(), like=dense)
         rand_ld = N.layout_of(rand_t)[1]
     N.check(N.lib().tf24_prune_compress(
-        dense.data_ptr(), N.dtype_code(dense.dtype), layout, ld, m, n, mode,
+        dense.data_ptr(), N.operand_code(dense.dtype), layout, ld, m, n, mode,
         N.ptr(mask_t), mask_code, mask_ld, N.ptr(rand_t), rand_ld,
-        values.data_ptr(), N.dtype_code(dtype), meta.data_ptr(),
+        values.data_ptr(), N.operand_code(dtype), meta.data_ptr(),
         N.COMPRESSED_PANEL if panel else N.COMPRESSED_CANONICAL, N.stream_ptr()))
     return values, meta
 
@@ -112,7 +123,7 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     # panel form once: the tiled kernel only streams that one.
     if (store_layout == N.COMPRESSED_CANONICAL and n >= 64 and dense.numel() // k >= 64 and k % _panel_width(values.dtype) == 0):
         pv, pm = torch.empty_like(values), torch.empty_like(meta)
-        N.check(N.lib().tf24_repack(values.data_ptr(), meta.data_ptr(), N.dtype_code(values.dtype), n, k, N.COMPRESSED_CANONICAL,
+        N.check(N.lib().tf24_repack(values.data_ptr(), meta.data_ptr(), N.operand_code(values.dtype), n, k, N.COMPRESSED_CANONICAL,
                                     pv.data_ptr(), pm.data_ptr(), N.stream_ptr()))
         sparse._set_storage(pv, pm, (n, k), N.COMPRESSED_PANEL)
         values, meta, store_layout = pv, pm, N.COMPRESSED_PANEL
@@ -145,17 +156,17 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     if kk != k:
         raise RuntimeError(f"inner dimensions do not match: sparse operand has k={k}, dense operand {tuple(dense.shape)}")
     if out_dtype is None:
-        out_dtype = torch.float32 if values.dtype in _FLOAT8 else values.dtype
+        out_dtype = torch.int32 if values.dtype == torch.int8 else torch.float32 if values.dtype in _FLOAT8 else values.dtype
     out = torch.empty(out_shape, dtype=out_dtype, device=dense.device)
     if bias is not None:
         bias = bias.to(out_dtype).contiguous()
         if bias.numel() != n:
             raise RuntimeError(f"bias must have {n} elements, got {bias.numel()}")
-    ws_bytes = N.lib().tf24_spmm_workspace_bytes(N.dtype_code(values.dtype), n, k, j)
+    ws_bytes = N.lib().tf24_spmm_workspace_bytes(N.operand_code(values.dtype), n, k, j)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dense.device) if ws_bytes else None
     N.check(N.lib().tf24_spmm(
-        values.data_ptr(), meta.data_ptr(), store_layout, N.dtype_code(values.dtype), n, k,
-        dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.dtype_code(out_dtype), c_layout, out.stride(0),
+        values.data_ptr(), meta.data_ptr(), store_layout, N.operand_code(values.dtype), n, k,
+        dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.operand_code(out_dtype), c_layout, out.stride(0),
         N.ptr(bias), float(scale), activation, N.ptr(workspace), ws_bytes, N.stream_ptr()))
     return out
 
@@ -362,7 +373,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
         values, meta = self._store_values, self._store_meta
         m, k = self._store_shape
         out = torch.empty((m, k), dtype=values.dtype, device=values.device)
-        N.check(N.lib().tf24_decompress(values.data_ptr(), N.dtype_code(values.dtype), meta.data_ptr(), self._store_layout,
+        N.check(N.lib().tf24_decompress(values.data_ptr(), N.operand_code(values.dtype), meta.data_ptr(), self._store_layout,
                                         m, k, out.data_ptr(), N.stream_ptr()))
         return out
 
@@ -393,8 +404,8 @@ def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = 
     `mask` (same shape, nonzero = keep) selects explicitly; `MVUE24=True` samples the
     minimum-variance unbiased estimator, taking its uniforms from `rand` (same shape, U[0,1);
     drawn with torch's generator when omitted).  `dtype` is the value dtype of the result
-    (float16, bfloat16, float8_e4m3fn or float8_e5m2).  Rows must be a multiple of 32, columns of 64
-    (128 for float8).  Same signature as the reference's factory (semi_structured.py:575-631)
+    (float16, bfloat16, float8_e4m3fn, float8_e5m2, or int8 for an int8 tensor).  Rows must be a
+    multiple of 32, columns of 64 (128 for 8-bit values).  Same signature as the reference's factory (semi_structured.py:575-631)
     plus `rand`.
     """
     return SparseSemiStructuredTensor(
@@ -417,7 +428,8 @@ def to_sparse_semi_structured_pair(original_tensor: torch.Tensor, mask: torch.Te
     if mask.dtype == torch.bool:
         mask = mask.view(torch.uint8)
     lay_w, lay_m = N.layout_of(w), N.layout_of(mask) if mask.dim() == 2 and mask.shape == w.shape else None
-    fits = (m >= unit and k >= unit and m % unit == 0 and k % unit == 0 and w.dtype in (torch.float32, torch.float16, torch.bfloat16)
+    fits = (m >= unit and k >= unit and m % unit == 0 and k % unit == 0 and ((w.dtype == torch.int8) == (dtype == torch.int8))
+            and w.dtype in (torch.float32, torch.float16, torch.bfloat16, torch.int8)
             and lay_w is not None and lay_m is not None and lay_w[0] == N.ROW_MAJOR and lay_m[0] == N.ROW_MAJOR
             and lay_w[1] % 8 == 0 and lay_m[1] % 8 == 0 and w.data_ptr() % 16 == 0 and mask.data_ptr() % 16 == 0
             and mask.dtype in N._DTYPES and SparseSemiStructuredTensor._PANEL_LAYOUT)
@@ -430,9 +442,9 @@ def to_sparse_semi_structured_pair(original_tensor: torch.Tensor, mask: torch.Te
     values, meta = buf[:half], buf[half:per].view(_indices_dtype(dtype))
     values_t, meta_t = buf[per:per + half], buf[per + half:].view(_indices_dtype(dtype))
     N.check(N.lib().tf24_prune_compress_dual(
-        w.data_ptr(), N.dtype_code(w.dtype), lay_w[1], m, k, mask.data_ptr(), N.dtype_code(mask.dtype), lay_m[1],
+        w.data_ptr(), N.operand_code(w.dtype), lay_w[1], m, k, mask.data_ptr(), N.dtype_code(mask.dtype), lay_m[1],
         values.data_ptr(), meta.data_ptr(), values_t.data_ptr(), meta_t.data_ptr(),
-        N.dtype_code(dtype), N.COMPRESSED_PANEL, N.stream_ptr()))
+        N.operand_code(dtype), N.COMPRESSED_PANEL, N.stream_ptr()))
     s = SparseSemiStructuredTensor._from_storage(values, meta, (m, k), N.COMPRESSED_PANEL, torch.Size((m, k)), False)
     s_t = SparseSemiStructuredTensor._from_storage(values_t, meta_t, (k, m), N.COMPRESSED_PANEL, torch.Size((k, m)), False)
     return s, s_t

@@ -43,7 +43,9 @@ typedef enum {
   TF24_BF16 = 2,
   TF24_E4M3 = 3, /* OCP float8 e4m3fn */
   TF24_E5M2 = 5, /* OCP float8 e5m2 (IEEE-like: infinities, NaN) */
-  TF24_U8 = 4    /* bytes: bool masks (nonzero = kept) */
+  TF24_U8 = 4,   /* bytes: bool masks (nonzero = kept) */
+  TF24_I8 = 6,   /* signed 8-bit integer values and operands (integer matmul, TF24_I32 results) */
+  TF24_I32 = 7   /* 32-bit integer matmul results and bias */
 } tf24_dtype;
 
 typedef enum { TF24_ROW_MAJOR = 0, TF24_COL_MAJOR = 1 } tf24_layout;
@@ -203,7 +205,10 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * Replaces sparse.cutlass.my_sparse_semi_structured_linear
  * (sparse/csrc/mySparseSemiStructuredLinear_cuda.cu:498-817, CUTLASS SparseGemm :61-76),
  * bound at sparse/sparse_semi_structured_linear.py:4-5.
- *   a_values, a_meta  the compressed operand in a_layout; dtype F16|BF16|E4M3|E5M2 (B has the same dtype)
+ *   a_values, a_meta  the compressed operand in a_layout; dtype F16|BF16|E4M3|E5M2|I8 (B has the same dtype).
+ *              I8 is the integer product of .cu:594-637: int32 accumulation, out_dtype and bias I32,
+ *              activation none or ReLU, scale 1; every other dtype accumulates in float32 and takes
+ *              out_dtype F16|BF16|F32 with a bias of that type
  *   b          dense operand, n_dense "columns" j: b_layout TF24_ROW_MAJOR means B is stored
  *              [n_dense, k] (k contiguous, element (k,j) at j*ldb + k: the X of X.W^T);
  *              TF24_COL_MAJOR means stored [k, n_dense] (element (k,j) at k*ldb + j)

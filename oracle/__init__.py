@@ -31,4 +31,4 @@ from .transposable import (  # noqa: F401
 from .decay import masked_add  # noqa: F401
 from .adamw import adamw_masked_decay  # noqa: F401
 from .gelu_glu import gelu_glu_forward, gelu_glu_backward  # noqa: F401
-from .spmm import spmm_ref, linear_ref  # noqa: F401
+from .spmm import spmm_ref, spmm_ref_int, linear_ref  # noqa: F401

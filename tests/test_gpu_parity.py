@@ -609,3 +609,90 @@ def test_spmm_tiled_k_strided_padded_rows(cuda, dtype):
     assert not xg.is_contiguous()
     out = torch.mm(s, xg)
     assert out.float().cpu().equal(ref.to(dtype).float())
+
+
+# ------------------------------------------------------------------ int8 values and the integer product
+def _int8(shape, seed, lo=-128, hi=128):
+    return torch.randint(lo, hi, shape, generator=torch.Generator().manual_seed(seed), dtype=torch.int64).to(torch.int8)
+
+
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("use_mask", [False, True])
+def test_int8_compress(cuda, col_major, use_mask):
+    """int8 dense -> int8 values + int32 metadata (semi_structured.py:24-30, 323-331): magnitude rule
+    on |x| with -128 the largest magnitude, ties to the larger index; masks as bytes or floats."""
+    import sparse
+    w = _int8((96, 384), 101)
+    w[:, :8] = torch.tensor([-128, 127, -127, 128 - 256, 5, -5, 5, -5], dtype=torch.int8)   # extremes and ties
+    mask = None
+    if use_mask:
+        _, mask = oracle.transposable_mask(w.float())
+        mask[:4] = torch.rand(4, 384, generator=torch.Generator().manual_seed(102)) < 0.5
+    want_v, want_m = oracle.compress24(w, mask=mask, out_dtype=torch.int8)
+    assert want_v.dtype == torch.int8 and want_m.dtype == torch.int32
+    for mk in ([None] if mask is None else [mask, mask.float()]):
+        s = sparse.to_sparse_semi_structured(maybe_t(w.to(cuda), col_major),
+                                             mask=None if mk is None else maybe_t(mk.to(cuda), col_major), dtype=torch.int8)
+        assert s.dtype == torch.int8
+        assert_same(s.values(), want_v, "values")
+        assert_same(s.indices(), want_m, "meta")
+        assert_same(s.to_dense(), oracle.decompress24(want_v, want_m), "to_dense")
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(w.to(cuda), dtype=torch.float16)          # int8 tensors give int8 values only
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(w.to(cuda).half(), dtype=torch.int8)
+    with pytest.raises(RuntimeError):
+        sparse.to_sparse_semi_structured(w.to(cuda), dtype=torch.int8, MVUE24=True)
+
+
+def test_int8_compress_pair(cuda):
+    import sparse
+    w = _int8((256, 128), 103)
+    _, mask = oracle.transposable_mask(w.float())
+    want_v, want_m = oracle.compress24(w, mask=mask, out_dtype=torch.int8)
+    want_vt, want_mt = oracle.compress24(w.t().contiguous(), mask=mask.t().contiguous(), out_dtype=torch.int8)
+    s, s_t = sparse.to_sparse_semi_structured_pair(w.to(cuda), mask.to(cuda), dtype=torch.int8)
+    assert_same(s.values(), want_v)
+    assert_same(s.indices(), want_m)
+    assert_same(s_t.values(), want_vt)
+    assert_same(s_t.indices(), want_mt)
+
+
+@pytest.mark.parametrize("dims", [(32, 128, 16), (64, 256, 40), (352, 640, 304), (256, 4096, 256), (96, 2048, 528)])
+def test_int8_spmm_is_exact(cuda, dims):
+    """int8 x int8 -> int32 (.cu:594-637) against an int64 product: general kernel, tiled kernel with
+    partial tiles, split-K; both operand positions and dense layouts; int32 bias and ReLU."""
+    import sparse
+    n, k, m = dims
+    w, x = _int8((n, k), 111), _int8((m, k), 112)
+    bias = torch.randint(-100000, 100000, (n,), generator=torch.Generator().manual_seed(113), dtype=torch.int64).int()
+    mask = oracle.prune24_mask(w.float())
+    wm = torch.where(mask, w, torch.zeros_like(w))
+    ref = oracle.spmm_ref_int(x, wm)
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=torch.int8)
+    xg = x.to(cuda)
+    out = torch.mm(xg, s.t())
+    assert out.dtype == torch.int32 and out.cpu().equal(ref)
+    assert torch.mm(maybe_t(xg, True), s.t()).cpu().equal(ref)                   # k strided dense operand
+    assert torch.mm(s, xg.t()).cpu().equal(ref.t())                              # sparse first
+    assert torch.mm(s, xg.t().contiguous()).cpu().equal(ref.t())
+    assert torch.addmm(bias.to(cuda), xg, s.t()).cpu().equal(oracle.spmm_ref_int(x, wm, bias))
+    out = sparse.sparse_semi_structured_linear(xg, s, bias=bias.to(cuda), activation="relu")
+    assert out.cpu().equal(oracle.spmm_ref_int(x, wm, bias, relu=True))
+    out = sparse.sparse_semi_structured_linear(xg, s.values(), s.indices())      # canonical pieces
+    assert out.cpu().equal(ref)
+    with pytest.raises(RuntimeError):
+        sparse.sparse_semi_structured_linear(xg, s, activation="silu")           # .cu:610-612: none and ReLU only
+    with pytest.raises(RuntimeError):
+        torch.mm(xg.half(), s.t())                                               # operand dtypes must match
+
+
+def test_int8_spmm_extreme_values(cuda):
+    """All operands -128: every product is +16384, the sum over k = 2048 kept pairs stays in int32."""
+    import sparse
+    n, k, m = 64, 4096, 64
+    w = torch.full((n, k), -128, dtype=torch.int8)
+    x = torch.full((m, k), -128, dtype=torch.int8)
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=torch.int8)
+    out = torch.mm(x.to(cuda), s.t())
+    assert out.cpu().equal(torch.full((m, n), 16384 * (k // 2), dtype=torch.int32))

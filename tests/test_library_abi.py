@@ -95,6 +95,27 @@ def test_transposable_and_spmm_validators(native):
     assert sp(N.F16, 32, 64, 8, act=5) == -5 and sp(N.F16, 32, 64, 8, bl=3) == -5
 
 
+def test_int8_validators(native):
+    """int8 values come from int8 matrices, take byte masks and no MVUE; the integer product gives
+    int32 with no activation or ReLU (.cu:594-637)."""
+    lib, N = native.lib(), native
+    pc = lambda **a: lib.tf24_prune_compress_validate(a.get("dt", N.I8), a.get("layout", N.ROW_MAJOR), a.get("ld", 128), 32, 128,
+                                                      a.get("mode", N.PRUNE_MAGNITUDE), a.get("has_mask", 0), a.get("mdt", N.U8),
+                                                      a.get("mld", 0), a.get("has_rand", 0), a.get("rld", 0), a.get("out", N.I8))
+    assert pc() == 0 and pc(mode=N.PRUNE_MASK, has_mask=1, mld=128) == 0
+    assert pc(out=N.F16) == -2 and pc(dt=N.F16) == -2                    # int8 <-> int8 only
+    assert pc(mode=N.PRUNE_MASK, has_mask=1, mld=128, mdt=N.F32) == -2   # byte masks only
+    assert pc(mode=N.PRUNE_MVUE, has_rand=1, rld=128) == -5
+    assert pc(layout=N.COL_MAJOR, ld=40) == -3 and pc(layout=N.COL_MAJOR, ld=48) == 0
+    sp = lambda **a: lib.tf24_spmm_validate(N.I8, 32, 128, N.ROW_MAJOR, 128, 16, a.get("out", N.I32), N.COL_MAJOR, 32, a.get("act", 0))
+    assert sp() == 0 and sp(act=N.ACT_RELU) == 0
+    assert sp(out=N.F32) == -2 and sp(act=N.ACT_SILU) == -5 and sp(act=N.ACT_GELU) == -5
+    assert lib.tf24_spmm_validate(N.F16, 32, 64, N.ROW_MAJOR, 64, 8, N.I32, N.COL_MAJOR, 32, 0) == -2
+    assert lib.tf24_prune_compress_dual_validate(N.I8, 128, 128, 128, N.U8, 128, N.I8, N.COMPRESSED_PANEL) == 0
+    assert lib.tf24_prune_compress_dual_validate(N.I8, 128, 128, 128, N.U8, 128, N.E4M3, N.COMPRESSED_PANEL) == -2
+    assert lib.tf24_prune_compress_dual_validate(N.I8, 64, 64, 64, N.U8, 64, N.I8, N.COMPRESSED_PANEL) == -1
+
+
 def test_dual_compress_validator(native):
     """Both W [m,k] and W^T [k,m] must be compressible: m and k multiples of 64 (128 for 8-bit values)."""
     lib, N = native.lib(), native
