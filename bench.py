@@ -25,7 +25,7 @@ import torch  # noqa: E402
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_DENSE_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA; SMFMAC executes MACs at this rate
 # HBM bytes per spmm launch (mean of forward and transposed) from two rocprofv3 --pmc runs of this file:
-# FETCH_SIZE 425399 KiB + WRITE_SIZE 120854 KiB, both counters reading factor 1.00 on a copy kernel of known size
+# FETCH_SIZE 424831 KiB + WRITE_SIZE 120846 KiB, both counters reading factor 1.00 on a copy kernel of known size
 SPMM_TRAFFIC_BYTES = (424831 + 120846) * 1024
 
 
