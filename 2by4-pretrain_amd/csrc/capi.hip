@@ -23,6 +23,12 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+int check_aligned(const char* fn, int bytes, std::initializer_list<const void*> ptrs) {
+  for (const void* p : ptrs)
+    if (p && (uintptr_t)p % (uintptr_t)bytes) return fail(TF24_ERR_STRIDE, "%s: pointer %p is not %d-byte aligned", fn, p, bytes);
+  return TF24_OK;
+}
+
 int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TF24_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));

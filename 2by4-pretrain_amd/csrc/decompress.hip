@@ -92,6 +92,8 @@ extern "C" int tf24_decompress(const void* values, int dtype, const void* meta, 
   const int64_t mult = is_8bit(dtype) ? 32 : 16;
   if (m <= 0 || k <= 0 || k % mult) return fail(TF24_ERR_SHAPE, "tf24_decompress: k=%lld must be a positive multiple of %lld", (long long)k, (long long)mult);
   if (!values || !meta || !dense_out) return fail(TF24_ERR_ARG, "tf24_decompress: null pointer");
+  if (int rc = check_aligned("tf24_decompress", 16, {values, dense_out})) return rc;
+  if (int rc = check_aligned("tf24_decompress", 8, {meta})) return rc;
   if (layout != TF24_COMPRESSED_CANONICAL && layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_decompress: bad compressed layout %d", layout);
   const bool panel = layout == TF24_COMPRESSED_PANEL;
   if (panel && k % (is_8bit(dtype) ? 128 : 64)) return fail(TF24_ERR_SHAPE, "tf24_decompress: panel layout needs whole panels (k=%lld)", (long long)k);

@@ -148,6 +148,7 @@ int run(const char* fn, const void* dense, int dtype, int layout, int64_t ld, in
   if (ld < extent || ld % 8) return fail(TF24_ERR_STRIDE, "%s: leading dimension %lld must be >= %lld and a multiple of 8", fn, (long long)ld, (long long)extent);
   if (OP == OP_MVUE && (!rnd || rand_ld < extent || rand_ld % 8)) return fail(TF24_ERR_ARG, "%s: rand tensor missing or bad leading dimension", fn);
   if (!dense || !sparse) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
+  if (int rc = check_aligned(fn, 16, {dense, sparse, mask, rnd})) return rc;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case TF24_F32: return launch<float, OP>(dense, layout, ld, m, k, rnd, rand_ld, sparse, mask, s, fn);

@@ -324,6 +324,8 @@ extern "C" int tf24_prune_compress(const void* dense, int in_dtype, int layout, 
                                         rnd != nullptr, rand_ld, out_dtype);
   if (rc != TF24_OK) return rc;
   if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "tf24_prune_compress: null dense/values/meta pointer");
+  if ((rc = check_aligned("tf24_prune_compress", 16, {dense, rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
+  if ((rc = check_aligned("tf24_prune_compress", 8, {meta, mask}))) return rc;
   if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
     return fail(TF24_ERR_ARG, "tf24_prune_compress: bad compressed layout %d", out_layout);
   const bool panel = out_layout == TF24_COMPRESSED_PANEL;

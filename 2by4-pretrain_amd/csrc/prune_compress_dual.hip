@@ -184,6 +184,8 @@ extern "C" int tf24_prune_compress_dual(const void* dense, int in_dtype, int64_t
   if (rc != TF24_OK) return rc;
   if (!dense || !mask || !values || !meta || !values_t || !meta_t)
     return fail(TF24_ERR_ARG, "tf24_prune_compress_dual: null dense/mask/values/meta pointer");
+  if ((rc = check_aligned("tf24_prune_compress_dual", 16, {dense, values, values_t, meta_t, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
+  if ((rc = check_aligned("tf24_prune_compress_dual", 8, {meta, mask}))) return rc;
   const bool panel = out_layout == TF24_COMPRESSED_PANEL;
   hipStream_t s = (hipStream_t)stream;
   switch (in_dtype) {

@@ -865,6 +865,9 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout,
   int rc = tf24_spmm_validate(dtype, n_sparse, k, b_layout, ldb, n_dense, out_dtype, c_layout, ldc, activation);
   if (rc) return rc;
   if (!a_values || !a_meta || !b || !c) return fail(TF24_ERR_ARG, "tf24_spmm: null pointer");
+  if ((rc = check_aligned("tf24_spmm", 16, {a_values, b, c, workspace}))) return rc;
+  if ((rc = check_aligned("tf24_spmm", 8, {a_meta}))) return rc;
+  if ((rc = check_aligned("tf24_spmm", dtype_size(out_dtype), {bias}))) return rc;
   if (a_layout != TF24_COMPRESSED_CANONICAL && a_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_spmm: bad compressed layout %d", a_layout);
   const bool panel = a_layout == TF24_COMPRESSED_PANEL;
   hipStream_t s = (hipStream_t)stream;

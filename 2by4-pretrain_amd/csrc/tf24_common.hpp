@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <initializer_list>
+
 #include "tf24.h"
 
 namespace tf24 {
@@ -11,6 +13,9 @@ namespace tf24 {
 void set_error(const char* fmt, ...);
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
+// TF24_ERR_STRIDE unless every listed pointer (NULL is skipped) is aligned to `bytes`: the kernels
+// use 128-bit (metadata and byte masks: 64-bit) accesses and do not handle split lines
+int check_aligned(const char* fn, int bytes, std::initializer_list<const void*> ptrs);
 
 // ---------------------------------------------------------------- element types
 struct f16_t { uint16_t bits; };

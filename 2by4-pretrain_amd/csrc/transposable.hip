@@ -196,6 +196,8 @@ extern "C" int tf24_transposable_mask(const void* dense, int dtype, int layout, 
   int rc = tf24_transposable_mask_validate(dtype, layout, ld, m, k);
   if (rc) return rc;
   if (!dense || !mask_out) return fail(TF24_ERR_ARG, "tf24_transposable_mask: null pointer");
+  if (int rc2 = check_aligned("tf24_transposable_mask", 16, {dense, sparse_out})) return rc2;
+  if (int rc2 = check_aligned("tf24_transposable_mask", 8, {mask_out})) return rc2;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case TF24_F32: return dispatch<float>(dense, layout, ld, m, k, use_abs, sparse_out, mask_out, s);

@@ -61,6 +61,7 @@ extern "C" int tf24_transpose(const void* in, int dtype, int64_t ld_in, int64_t 
   if (ld_in < cols || ld_in % v || ld_out < rows || ld_out % v)
     return fail(TF24_ERR_STRIDE, "tf24_transpose: leading dimensions must cover the rows and be multiples of %lld", (long long)v);
   if (!in || !out) return fail(TF24_ERR_ARG, "tf24_transpose: null pointer");
+  if (int rc = check_aligned("tf24_transpose", 16, {in, out})) return rc;
   hipStream_t s = (hipStream_t)stream;
   if (es == 2) return launch<uint16_t>(in, ld_in, rows, cols, out, ld_out, s);
   return launch<uint8_t>(in, ld_in, rows, cols, out, ld_out, s);

@@ -95,6 +95,24 @@ def test_transposable_and_spmm_validators(native):
     assert sp(N.F16, 32, 64, 8, act=5) == -5 and sp(N.F16, 32, 64, 8, bl=3) == -5
 
 
+def test_misaligned_pointers_are_refused_before_any_launch(native):
+    """The kernels use 128-bit accesses: entry points return TF24_ERR_STRIDE for a misaligned
+    pointer instead of launching (no GPU is touched on this path, the addresses are made up)."""
+    lib, N = native.lib(), native
+    ok, off = 0x7f0000001000, 0x7f0000001008
+    spmm = lambda a=ok, b=ok, c=ok, meta=ok: lib.tf24_spmm(a, meta, N.COMPRESSED_PANEL, N.F16, 64, 64, b, N.ROW_MAJOR, 64, 64,
+                                                           c, N.F16, N.COL_MAJOR, 64, None, 1.0, 0, None, 0, None)
+    assert spmm(b=off) == -3 and spmm(a=off) == -3 and spmm(c=off) == -3 and spmm(meta=ok + 4) == -3
+    assert b"aligned" in lib.tf24_last_error()
+    pc = lambda dense=ok, values=ok: lib.tf24_prune_compress(dense, N.F16, N.ROW_MAJOR, 64, 32, 64, N.PRUNE_MAGNITUDE, None, N.U8, 0,
+                                                             None, 0, values, N.F16, ok, N.COMPRESSED_PANEL, None)
+    assert pc(dense=off) == -3 and pc(values=off) == -3
+    assert lib.tf24_transposable_mask(off, N.F16, N.ROW_MAJOR, 64, 32, 64, 1, None, ok, None) == -3
+    assert lib.tf24_soft_threshold24(ok, N.F16, N.ROW_MAJOR, 64, 32, 64, off, ok, None) == -3
+    assert lib.tf24_transpose(ok, N.F16, 64, 64, 64, off, 64, None) == -3
+    assert lib.tf24_decompress(off, N.F16, ok, N.COMPRESSED_CANONICAL, 32, 64, ok, None) == -3
+
+
 def test_int8_validators(native):
     """int8 values come from int8 matrices, take byte masks and no MVUE; the integer product gives
     int32 with no activation or ReLU (.cu:594-637)."""
