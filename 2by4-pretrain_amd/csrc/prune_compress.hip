@@ -135,7 +135,8 @@ __global__ void __launch_bounds__(kThreads)
 prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel, bool rand_packed) {
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel, bool rand_packed,
+                   float* __restrict__ rowsum_partial) {
   constexpr int R = 16 / sizeof(In);
   constexpr int TR = 8 * R;          // tile rows
   constexpr int TC = 128;            // tile columns (32 groups)
@@ -143,12 +144,20 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
   constexpr int MPITCH = TC / 8 + 4;                   // bytes per row of the metadata tile
   __shared__ __attribute__((aligned(16))) uint8_t s_val[TR * VPITCH];
   __shared__ __attribute__((aligned(16))) uint8_t s_meta[TR * MPITCH];
+  // Row sums of the dense input (the bias gradient when the input is dY^T): a lane adds its 4
+  // columns, the 32 lanes that share a row meet in LDS, the block leaves one float per row in
+  // rowsum_partial[column block][row]; a second kernel adds the column blocks.  Fixed order throughout.
+  constexpr int SPITCH = TC / 4 + 1;
+  __shared__ float s_sum[TR * SPITCH];
 
   const int tid = threadIdx.x;
   const int rchunk = tid & 7, grp = tid >> 3;           // 8 row chunks x 32 groups
   // consecutive blockIdx.x walk the contiguous (row) dimension of the column-major input
   const int64_t row0 = (int64_t)blockIdx.x * TR, col0 = (int64_t)blockIdx.y * TC;
   const int64_t r0 = row0 + rchunk * R, c0 = col0 + grp * 4;
+  float psum[R];
+#pragma unroll
+  for (int i = 0; i < R; i++) psum[i] = 0.0f;
   if (r0 < m && c0 < k) {
     Pack<In, R> in[4];
     Pack<MaskT, R> mk[4];
@@ -173,6 +182,7 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       for (int c = 0; c < 4; c++) { x[c] = to_float(in[c].v[i]); if constexpr (MODE == TF24_PRUNE_MASK) mrow[c] = mk[c].v[i]; }
       float u0 = 0.f, u1 = 0.f;
       if constexpr (MODE == TF24_PRUNE_MVUE) { u0 = rr[0].v[i]; u1 = rr[1].v[i]; }
+      if (rowsum_partial) psum[i] = (x[0] + x[1]) + (x[2] + x[3]);
       uint32_t mb = prune_group<In, MODE, MaskT>(x, mrow, u0, u1, pr);
       uint32_t nib = encode_nibble(mb);
       Pack<Out, 2> o;
@@ -185,7 +195,16 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       if ((grp & 1) == 0) s_meta[lr * MPITCH + (grp >> 1)] = (uint8_t)(nib | (other << 4));
     }
   }
+  if (rowsum_partial) {
+#pragma unroll
+    for (int i = 0; i < R; i++) s_sum[(rchunk * R + i) * SPITCH + grp] = psum[i];
+  }
   __syncthreads();
+  if (rowsum_partial && tid < TR && row0 + tid < m) {
+    float t = 0.0f;
+    for (int g = 0; g < TC / 4; g++) t += s_sum[tid * SPITCH + g];
+    rowsum_partial[(int64_t)blockIdx.y * m + row0 + tid] = t;
+  }
   // values: TR rows x (TC/2)*sizeof(Out) bytes, 16 bytes per lane.  Canonical output: row gr, byte
   // offset (col0/2)*sizeof(Out) + seg*16 of a k/2-element row.  Panel output: the tile covers
   // TC/KP panels (KP = 128/sizeof(Out) dense columns, 64 bytes of values per row); panel p of row gr
@@ -237,9 +256,31 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
   }
 }
 
+// rowsum[r] = sum over column blocks of partial[b][r], one rounding to T.  A block takes 32 rows;
+// its 8 groups of 32 lanes each add every 8th column block (coalesced 128-byte reads), then the 8
+// group sums of a row are added in group order.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+rowsum_finish(const float* __restrict__ partial, int nblocks, int64_t m, T* __restrict__ out) {
+  __shared__ float s_part[8][32];
+  const int lr = threadIdx.x & 31, part = threadIdx.x >> 5;
+  const int64_t r = (int64_t)blockIdx.x * 32 + lr;
+  float t = 0.0f;
+  if (r < m)
+    for (int b = part; b < nblocks; b += 8) t += partial[(int64_t)b * m + r];
+  s_part[part][lr] = t;
+  __syncthreads();
+  if (part == 0 && r < m) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; q++) sum += s_part[q][lr];
+    out[r] = from_float<T>(sum);
+  }
+}
+
 template <typename In, typename Out, int MODE, typename MaskT>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
-           const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t stream) {
+           const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t stream) {
   if (layout == TF24_ROW_MAJOR) {
     const int64_t per_block = kThreads * kUnroll;
     const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == (rand_packed ? k / 2 : k));
@@ -259,26 +300,27 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
     constexpr int R = 16 / sizeof(In);
     dim3 grid((unsigned)((m + 8 * R - 1) / (8 * R)), (unsigned)((k + 127) / 128));
     hipLaunchKernelGGL((prune_compress_col<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
-                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel, rand_packed);
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel, rand_packed,
+                       rowsum_partial);
   }
   return check_launch("tf24_prune_compress");
 }
 
 template <typename In, typename Out, int MODE>
 int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int mask_dtype,
-                  int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
+                  int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
   if constexpr (MODE != TF24_PRUNE_MASK) {
-    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
   } else if constexpr (std::is_same<In, i8_t>::value) {
     // int8 matrices take byte masks only (the column kernel reads 16 rows per lane: 16-byte mask loads)
     if (mask_dtype != TF24_U8) return fail(TF24_ERR_DTYPE, "tf24_prune_compress: int8 input takes a byte mask (dtype %d given)", mask_dtype);
-    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
   } else {
     switch (mask_dtype) {
-      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
     }
     return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported mask dtype %d", mask_dtype);
   }
@@ -286,30 +328,59 @@ int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t 
 
 template <typename In, typename Out>
 int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
+                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
   switch (mode) {
     case TF24_PRUNE_MAGNITUDE:
-      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
     case TF24_PRUNE_MASK:
-      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
     case TF24_PRUNE_MVUE:
     case TF24_PRUNE_MVUE_PACKED:
       if constexpr (std::is_same<Out, i8_t>::value) break;        // refused by the validator
-      else return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+      else return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
   }
   return fail(TF24_ERR_ARG, "tf24_prune_compress: bad mode %d", mode);
 }
 
 template <typename In>
 int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, hipStream_t s) {
+                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
   switch (out_dtype) {
-    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported output dtype %d", out_dtype);
+}
+
+}  // namespace
+}  // namespace tf24
+
+namespace tf24 {
+namespace {
+
+int run_prune_compress(const char* fn, const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                       int mode, const void* mask, int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld,
+                       void* values, int out_dtype, void* meta, int out_layout, float* rowsum_partial, void* stream) {
+  int rc = tf24_prune_compress_validate(in_dtype, layout, ld, m, k, mode, mask != nullptr, mask_dtype, mask_ld,
+                                        rnd != nullptr, rand_ld, out_dtype);
+  if (rc != TF24_OK) return rc;
+  if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "%s: null dense/values/meta pointer", fn);
+  if ((rc = check_aligned(fn, 16, {dense, rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
+  if ((rc = check_aligned(fn, 8, {meta, mask}))) return rc;
+  if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
+    return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, out_layout);
+  const bool panel = out_layout == TF24_COMPRESSED_PANEL;
+  const bool rand_packed = mode == TF24_PRUNE_MVUE_PACKED;
+  hipStream_t s = (hipStream_t)stream;
+  switch (in_dtype) {
+    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_I8: return dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+  }
+  return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
 }
 
 }  // namespace
@@ -319,23 +390,43 @@ extern "C" int tf24_prune_compress(const void* dense, int in_dtype, int layout, 
                                    int mode, const void* mask, int mask_dtype, int64_t mask_ld,
                                    const float* rnd, int64_t rand_ld,
                                    void* values, int out_dtype, void* meta, int out_layout, void* stream) {
+  return tf24::run_prune_compress("tf24_prune_compress", dense, in_dtype, layout, ld, m, k, mode, mask, mask_dtype, mask_ld, rnd, rand_ld,
+                                  values, out_dtype, meta, out_layout, nullptr, stream);
+}
+
+extern "C" int64_t tf24_prune_compress_rowsum_workspace_bytes(int64_t m, int64_t k) {
+  return m > 0 && k > 0 ? ((k + 127) / 128) * m * (int64_t)sizeof(float) : 0;
+}
+
+extern "C" int tf24_prune_compress_rowsum(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                                          int mode, const void* mask, int mask_dtype, int64_t mask_ld,
+                                          const float* rnd, int64_t rand_ld,
+                                          void* values, int out_dtype, void* meta, int out_layout,
+                                          void* rowsum, int rowsum_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
   using namespace tf24;
-  int rc = tf24_prune_compress_validate(in_dtype, layout, ld, m, k, mode, mask != nullptr, mask_dtype, mask_ld,
-                                        rnd != nullptr, rand_ld, out_dtype);
-  if (rc != TF24_OK) return rc;
-  if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "tf24_prune_compress: null dense/values/meta pointer");
-  if ((rc = check_aligned("tf24_prune_compress", 16, {dense, rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
-  if ((rc = check_aligned("tf24_prune_compress", 8, {meta, mask}))) return rc;
-  if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
-    return fail(TF24_ERR_ARG, "tf24_prune_compress: bad compressed layout %d", out_layout);
-  const bool panel = out_layout == TF24_COMPRESSED_PANEL;
-  const bool rand_packed = mode == TF24_PRUNE_MVUE_PACKED;
+  const char* fn = "tf24_prune_compress_rowsum";
+  if (layout != TF24_COL_MAJOR)
+    return fail(TF24_ERR_ARG, "%s: row sums are produced for column-major input only (a row of a row-major matrix is contiguous: sum it directly)", fn);
+  if (in_dtype == TF24_I8) return fail(TF24_ERR_DTYPE, "%s: int8 input is not supported", fn);
+  if (rowsum_dtype != TF24_F32 && rowsum_dtype != TF24_F16 && rowsum_dtype != TF24_BF16)
+    return fail(TF24_ERR_DTYPE, "%s: unsupported row-sum dtype %d", fn, rowsum_dtype);
+  if (!rowsum || !workspace) return fail(TF24_ERR_ARG, "%s: null rowsum/workspace pointer", fn);
+  if (workspace_bytes < tf24_prune_compress_rowsum_workspace_bytes(m, k))
+    return fail(TF24_ERR_ARG, "%s: workspace of %lld bytes is too small (%lld needed)", fn, (long long)workspace_bytes,
+                (long long)tf24_prune_compress_rowsum_workspace_bytes(m, k));
+  int rc = check_aligned(fn, 4, {workspace});
+  if (rc) return rc;
+  if ((rc = check_aligned(fn, dtype_size(rowsum_dtype), {rowsum}))) return rc;
+  rc = run_prune_compress(fn, dense, in_dtype, layout, ld, m, k, mode, mask, mask_dtype, mask_ld, rnd, rand_ld, values, out_dtype, meta,
+                          out_layout, (float*)workspace, stream);
+  if (rc) return rc;
+  const int nblocks = (int)((k + 127) / 128);
+  dim3 grid((unsigned)((m + 31) / 32));
   hipStream_t s = (hipStream_t)stream;
-  switch (in_dtype) {
-    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
-    case TF24_I8: return dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, s);
+  switch (rowsum_dtype) {
+    case TF24_F32: hipLaunchKernelGGL((rowsum_finish<float>), grid, dim3(kThreads), 0, s, (const float*)workspace, nblocks, m, (float*)rowsum); break;
+    case TF24_F16: hipLaunchKernelGGL((rowsum_finish<f16_t>), grid, dim3(kThreads), 0, s, (const float*)workspace, nblocks, m, (f16_t*)rowsum); break;
+    default: hipLaunchKernelGGL((rowsum_finish<bf16_t>), grid, dim3(kThreads), 0, s, (const float*)workspace, nblocks, m, (bf16_t*)rowsum); break;
   }
-  return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported input dtype %d", in_dtype);
+  return check_launch(fn);
 }

@@ -4,7 +4,8 @@ Same names as the reference package (sparse/__init__.py:1-25) for everything on 
 every operator runs a hand-written HIP kernel from lib2by4_gfx950.so and raises if that library
 is missing -- there is no CPU or PyTorch fallback.
 """
-from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair
+from .semi_structured import (SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair,
+                              to_sparse_semi_structured_with_row_sums)
 from .transposable_semi_structured import TransposableSparse, mask_select
 from .decay import masked_add_
 from .adamw import MaskedDecayAdamW
@@ -17,6 +18,7 @@ from .sparse_ops import MyLinear, SparseLinear, SoftThreshold, SoftThresholdLine
 
 __all__ = [
     "SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair",
+    "to_sparse_semi_structured_with_row_sums",
     "TransposableSparse", "mask_select",
     "masked_add_", "MaskedDecayAdamW",
     "soft_threshold24", "sparse24", "MVUE24_approx",

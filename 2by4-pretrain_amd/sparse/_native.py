@@ -34,6 +34,8 @@ _SIGNATURES = {
     "tf24_last_error": (ctypes.c_char_p, []),
     "tf24_prune_compress": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p]),
     "tf24_prune_compress_validate": (_i, [_i, _i, _i64, _i64, _i64, _i, _i, _i, _i64, _i, _i64, _i]),
+    "tf24_prune_compress_rowsum": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p, _i, _p, _i64, _p]),
+    "tf24_prune_compress_rowsum_workspace_bytes": (_i64, [_i64, _i64]),
     "tf24_prune_compress_dual": (_i, [_p, _i, _i64, _i64, _i64, _p, _i, _i64, _p, _p, _p, _p, _i, _i, _p]),
     "tf24_prune_compress_dual_validate": (_i, [_i, _i64, _i64, _i64, _i, _i64, _i, _i]),
     "tf24_decompress": (_i, [_p, _i, _p, _i, _i64, _i64, _p, _p]),

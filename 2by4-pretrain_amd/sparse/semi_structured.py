@@ -22,7 +22,8 @@ import torch
 
 from . import _native as N
 
-__all__ = ["SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair"]
+__all__ = ["SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair",
+           "to_sparse_semi_structured_with_row_sums"]
 
 _Config = namedtuple("_SEMI_STRUCTURED_SPARSE_CONFIG",
                      "compression_factor sparse_min_rows sparse_min_cols dense_min_rows dense_min_cols")
@@ -61,9 +62,10 @@ def _to_canonical(values, meta, m, n):
     return v, mt
 
 
-def _compress(original, dtype, MVUE24, mask, rand, panel):
+def _compress(original, dtype, MVUE24, mask, rand, panel, row_sums=False):
     """One allocation of numel*cf/16 elements: values first, metadata in the tail
-    (reference :215-243); then the HIP prune+compress kernel.  Returns flat storage views."""
+    (reference :215-243); then the HIP prune+compress kernel.  Returns flat storage views; with
+    `row_sums` (column-major input only) also original.sum(1), taken from the same read."""
     m, n = original.shape
     cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[dtype]
     buf = torch.empty((original.nelement() * cfg.compression_factor // 16,), dtype=dtype, device=original.device)
@@ -106,6 +108,17 @@ def _compress(original, dtype, MVUE24, mask, rand, panel):
                                f"(or its packed form {(m, n // 2)})")
         rand_t = N.as_matrix(rand.float(), like=dense)
         rand_ld = N.layout_of(rand_t)[1]
+    if row_sums:
+        sums = torch.empty((m,), dtype=dense.dtype, device=dense.device)
+        ws_bytes = N.lib().tf24_prune_compress_rowsum_workspace_bytes(m, n)
+        workspace = torch.empty((ws_bytes // 4,), dtype=torch.float32, device=dense.device)
+        N.check(N.lib().tf24_prune_compress_rowsum(
+            dense.data_ptr(), N.operand_code(dense.dtype), layout, ld, m, n, mode,
+            N.ptr(mask_t), mask_code, mask_ld, N.ptr(rand_t), rand_ld,
+            values.data_ptr(), N.operand_code(dtype), meta.data_ptr(),
+            N.COMPRESSED_PANEL if panel else N.COMPRESSED_CANONICAL,
+            sums.data_ptr(), N.dtype_code(sums.dtype), workspace.data_ptr(), ws_bytes, N.stream_ptr()))
+        return values, meta, sums
     N.check(N.lib().tf24_prune_compress(
         dense.data_ptr(), N.operand_code(dense.dtype), layout, ld, m, n, mode,
         N.ptr(mask_t), mask_code, mask_ld, N.ptr(rand_t), rand_ld,
@@ -448,3 +461,28 @@ def to_sparse_semi_structured_pair(original_tensor: torch.Tensor, mask: torch.Te
     s = SparseSemiStructuredTensor._from_storage(values, meta, (m, k), N.COMPRESSED_PANEL, torch.Size((m, k)), False)
     s_t = SparseSemiStructuredTensor._from_storage(values_t, meta_t, (k, m), N.COMPRESSED_PANEL, torch.Size((k, m)), False)
     return s, s_t
+
+
+def to_sparse_semi_structured_with_row_sums(original_tensor: torch.Tensor, MVUE24: bool = False,
+                                            mask: Optional[torch.Tensor] = None, dtype: torch.dtype = torch.float16,
+                                            rand: Optional[torch.Tensor] = None):
+    """(to_sparse_semi_structured(t, MVUE24=..., mask=..., dtype=..., rand=...), t.sum(1)).
+
+    For a column-major `t` (the `grad_output.t()` of the training layer's backward, README.md:190-197,
+    where the row sums are the bias gradient `grad_output.sum(0)`) both results come from one pass over
+    `t`; the sums are added in float32 and rounded once to t's dtype.  Any other input runs the
+    conversion and torch's sum separately."""
+    t = original_tensor
+    cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG.get(dtype)
+    fusable = (t.is_cuda and t.dim() == 2 and cfg is not None and t.dtype in (torch.float32, torch.float16, torch.bfloat16)
+               and dtype != torch.int8 and not (mask is not None and MVUE24) and SparseSemiStructuredTensor._PANEL_LAYOUT)
+    if fusable:
+        m, n = t.shape
+        lay = N.layout_of(t)
+        fusable = (m >= cfg.sparse_min_rows and m % cfg.sparse_min_rows == 0 and n >= cfg.sparse_min_cols
+                   and n % cfg.sparse_min_cols == 0 and lay is not None and lay[0] == N.COL_MAJOR and lay[1] % 8 == 0
+                   and t.data_ptr() % 16 == 0 and t.stride(0) == 1)
+    if not fusable:
+        return (to_sparse_semi_structured(t, MVUE24=MVUE24, mask=mask, dtype=dtype, rand=rand), t.sum(1))
+    values, meta, sums = _compress(t, dtype, MVUE24, mask, rand, True, row_sums=True)
+    return SparseSemiStructuredTensor._from_storage(values, meta, (m, n), N.COMPRESSED_PANEL, torch.Size((m, n)), False), sums

@@ -15,7 +15,8 @@ import torch.nn.functional as F
 from torch import autograd, nn
 from torch.amp import custom_bwd, custom_fwd
 
-from .semi_structured import SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair
+from .semi_structured import (SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair,
+                              to_sparse_semi_structured_with_row_sums)
 from .transposable_semi_structured import TransposableSparse
 
 __all__ = ["SparseLinearTranspose", "sparse_linear_transpose"]
@@ -46,8 +47,13 @@ class sparse_linear_transpose(autograd.Function):
             grad_input = torch.mm(grad_output, weight_T.t()).view(ctx.shape)
         if ctx.needs_input_grad[1]:
             input = input.view(-1, input.shape[-1])
-            grad_weight = torch.mm(to_sparse_semi_structured(grad_output.t(), MVUE24=True, dtype=grad_output.dtype), input)
-        if ctx.needs_input_grad[4]:
+            if ctx.needs_input_grad[4]:
+                # MVUE24(dY^T) and grad_bias = dY.sum(0) (README.md:193-197) from one read of dY
+                grad_sparse, grad_bias = to_sparse_semi_structured_with_row_sums(grad_output.t(), MVUE24=True, dtype=grad_output.dtype)
+            else:
+                grad_sparse = to_sparse_semi_structured(grad_output.t(), MVUE24=True, dtype=grad_output.dtype)
+            grad_weight = torch.mm(grad_sparse, input)
+        elif ctx.needs_input_grad[4]:
             grad_bias = grad_output.sum(0)
         return grad_input, grad_weight, None, None, grad_bias
 

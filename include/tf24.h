@@ -100,6 +100,26 @@ int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld,
                         void* values, int out_dtype, void* meta, int out_layout, void* stream);
 
 /*
+ * tf24_prune_compress of a column-major matrix that also returns its row sums,
+ *     rowsum[r] = sum_c dense[r, c]   (the unpruned input, added in float32, one rounding to rowsum_dtype).
+ * Replaces the pair the training layer's backward issues on the same gradient (README.md:190-197):
+ *     to_sparse_semi_structured(grad_output.t(), MVUE24=True)   and   grad_bias = grad_output.sum(0)
+ * -- with dense = grad_output^T (column-major view) the row sums are the bias gradient, from the read
+ * the compression makes anyway.  Arguments as tf24_prune_compress, plus
+ *   rowsum     m elements of rowsum_dtype (F32|F16|BF16)
+ *   workspace  tf24_prune_compress_rowsum_workspace_bytes(m, k) bytes of float32 scratch (one partial
+ *              sum per row and block of 128 columns; added in a fixed order: deterministic)
+ * layout must be TF24_COL_MAJOR (a row of a row-major matrix is contiguous and needs no fusion);
+ * int8 input is not supported.
+ */
+int tf24_prune_compress_rowsum(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                               int mode, const void* mask, int mask_dtype, int64_t mask_ld,
+                               const float* rand, int64_t rand_ld,
+                               void* values, int out_dtype, void* meta, int out_layout,
+                               void* rowsum, int rowsum_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+int64_t tf24_prune_compress_rowsum_workspace_bytes(int64_t m, int64_t k);
+
+/*
  * Mask-driven 2:4 compression of W and of W^T from ONE read of W and of the mask:
  *   (values, meta)      = tf24_prune_compress(W   [m,k] row-major,          mode MASK, mask)
  *   (values_t, meta_t)  = tf24_prune_compress(W^T [k,m] (W read by columns), mode MASK, mask^T)

@@ -202,6 +202,56 @@ def test_mask_compress_pair_falls_back_and_rejects(cuda):
     assert lib.tf24_prune_compress_dual_validate(N.U8, 128, 128, 128, N.U8, 128, N.F16, N.COMPRESSED_PANEL) != 0
 
 
+@pytest.mark.parametrize("mode", ["magnitude", "mvue"])
+@pytest.mark.parametrize("dtype,shape", [(F16, (96, 320)), (BF16, (64, 128)), (F32, (160, 192)), (F16, (3072, 1024))])
+def test_compress_with_row_sums(cuda, dtype, shape, mode):
+    """Compression of a column-major matrix that also returns its row sums (the bias gradient when the
+    matrix is dY^T): compressed bytes identical to the plain conversion, sums within float32
+    accumulation error of the exact sum and one rounding to the input dtype."""
+    import sparse
+    from sparse import _native as N
+    m, k = shape
+    t = randn((k, m), dtype, 19).t()                             # [m, k] column-major
+    rand = torch.rand((k // 2, m), generator=torch.Generator().manual_seed(20)).t() if mode == "mvue" else None
+    kw = dict(MVUE24=mode == "mvue", dtype=F16, rand=None if rand is None else rand.to(cuda))
+    plain = sparse.to_sparse_semi_structured(t.to(cuda), **kw)
+    fused, sums = sparse.to_sparse_semi_structured_with_row_sums(t.to(cuda), **kw)
+    assert fused._store_layout == N.COMPRESSED_PANEL
+    assert_same(fused.values(), plain.values().cpu(), "values")
+    assert_same(fused.indices(), plain.indices().cpu(), "meta")
+    want = t.double().sum(1)
+    assert sums.shape == (m,) and sums.dtype == dtype
+    eps = {F16: 2.0 ** -11, BF16: 2.0 ** -8, F32: 2.0 ** -24}[dtype]
+    tol = eps * want.abs() + 2e-7 * (k ** 0.5) * t.double().abs().sum(1) / k ** 0.5 + 1e-30
+    assert ((sums.double().cpu() - want).abs() <= tol + eps * want.abs().max()).all()
+    # deterministic: the same bits every time
+    again = sparse.to_sparse_semi_structured_with_row_sums(t.to(cuda), **kw)[1]
+    assert again.equal(sums)
+
+
+def test_compress_with_row_sums_other_layouts(cuda):
+    """Row-major input runs the two operations separately; the C entry point refuses it."""
+    import sparse
+    from sparse import _native as N
+    t = randn((64, 128), F16, 21)
+    s, sums = sparse.to_sparse_semi_structured_with_row_sums(t.to(cuda))
+    want_v, want_m = oracle.compress24(t)
+    assert_same(s.values(), want_v)
+    assert_same(s.indices(), want_m)
+    assert torch.allclose(sums.float().cpu(), t.float().sum(1), rtol=2e-3, atol=2e-2)
+    d = t.to(cuda)
+    v = torch.empty(64 * 64, dtype=F16, device=cuda)
+    mt = torch.empty(64 * 16, dtype=torch.uint8, device=cuda)
+    out = torch.empty(64, dtype=F16, device=cuda)
+    ws = torch.empty(64, dtype=torch.float32, device=cuda)
+    call = lambda layout, ws_bytes: N.lib().tf24_prune_compress_rowsum(
+        d.data_ptr(), N.F16, layout, 128, 64, 128, N.PRUNE_MAGNITUDE, None, N.U8, 0, None, 0, v.data_ptr(), N.F16, mt.data_ptr(),
+        N.COMPRESSED_PANEL, out.data_ptr(), N.F16, ws.data_ptr(), ws_bytes, N.stream_ptr())
+    assert call(N.ROW_MAJOR, 256) == -5
+    assert N.lib().tf24_prune_compress_rowsum_workspace_bytes(64, 128) == 256
+    assert N.lib().tf24_prune_compress_rowsum_workspace_bytes(3072, 12288) == 96 * 3072 * 4
+
+
 def test_mask_layout_mismatch_is_copied(cuda):
     import sparse
     w = randn((64, 128), F16, 14)
