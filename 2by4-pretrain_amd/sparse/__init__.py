@@ -9,6 +9,7 @@ from .semi_structured import (SparseSemiStructuredTensor, to_sparse_semi_structu
 from .transposable_semi_structured import TransposableSparse, mask_select
 from .decay import masked_add_
 from .adamw import MaskedDecayAdamW
+from .adamw_step import AdamW_STEP
 from .dense_ops import (soft_threshold24, sparse24, MVUE24_approx,
                         soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton)
 from .sparse_linear_transpose import SparseLinearTranspose, sparse_linear_transpose
@@ -20,7 +21,7 @@ __all__ = [
     "SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair",
     "to_sparse_semi_structured_with_row_sums",
     "TransposableSparse", "mask_select",
-    "masked_add_", "MaskedDecayAdamW",
+    "masked_add_", "MaskedDecayAdamW", "AdamW_STEP",
     "soft_threshold24", "sparse24", "MVUE24_approx",
     "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
     "SparseLinearTranspose", "sparse_linear_transpose",

@@ -49,6 +49,8 @@ _SIGNATURES = {
     "tf24_adamw_masked_decay": (_i, [_p, _p, _i, _p, _p, _p, _i, _i64, _d, _d, _d, _d, _d, _d, _i64, _p]),
     "tf24_gelu_glu_forward": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _i64, _p]),
     "tf24_gelu_glu_backward": (_i, [_p, _i64, _p, _i, _i, _i64, _i64, _i64, _p, _i64, _p]),
+    "tf24_adamw_step": (_i, [_p, _p, _i, _p, _p, _p, _p, _i64, _d, _d, _d, _d, _d, _i64, _p, _i, _p]),
+    "tf24_adamw_step_partials": (_i64, [_i64]),
     "tf24_spmm": (_i, [_p, _p, _i, _i, _i64, _i64, _p, _i, _i64, _i64, _p, _i, _i, _i64, _p, _f, _i, _p, _i64, _p]),
     "tf24_spmm_workspace_bytes": (_i64, [_i, _i64, _i64, _i64]),
     "tf24_transpose": (_i, [_p, _i, _i64, _i64, _i64, _p, _i64, _p]),

@@ -211,6 +211,27 @@ int tf24_adamw_masked_decay(float* p, const void* grad, int grad_dtype, float* e
                             double eps, double weight_decay, double decay_alpha, int64_t step, void* stream);
 
 /*
+ * The update of the STEP optimizer, one pass per tensor: replaces the body of AdamW_STEP.step
+ * (sparse/adamw_step.py:84-148; the recipe is README.md:271-329).  Decoupled weight decay and the two
+ * moments as in AdamW; then
+ *   phase 1 (precond_variance == NULL): denom = sqrt(v) / sqrt(bc2) + eps, of max(max_exp_avg_sq, v)
+ *            when max_exp_avg_sq is given (amsgrad; updated in place);
+ *   phase 2 (precond_variance given: the variance frozen when the optimizer switched phases, :186-194):
+ *            denom = sqrt(precond_variance) + eps^(3/4)                               (:131-135)
+ *   p += -(lr / bc1) * exp_avg / denom.
+ * z_option 1 | 2 with z_partial: the terms |v_t - v_{t-1}| (1) or log|v_t - v_{t-1}| (2) of the
+ * variance-change statistic Z_t (:124-129, :152-158) are summed per block of 1024 elements into
+ * z_partial[0 .. tf24_adamw_step_partials(n)); the caller adds the partial sums of all tracked
+ * tensors and divides by their element count (option 2: then exponentiates).  z_option 0 and
+ * z_partial NULL: no statistic.  p, moments, precond_variance float32; grad F32|F16|BF16; step >= 1.
+ */
+int tf24_adamw_step(float* p, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
+                    float* max_exp_avg_sq, const float* precond_variance, int64_t n,
+                    double lr, double beta1, double beta2, double eps, double weight_decay, int64_t step,
+                    float* z_partial, int z_option, void* stream);
+int64_t tf24_adamw_step_partials(int64_t n);
+
+/*
  * Masked decay, in place: grad[i] += alpha * p[i] where mask[i] == 0.
  * Replaces masked_add_kernel / masked_add_ (sparse/decay.py:7-37).  Flat over n elements
  * (the reference requires identical strides and indexes storage linearly).

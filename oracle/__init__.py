@@ -15,6 +15,7 @@ Pinning status (what fixes each function independently of this file):
   transposable_mask      90-way fp64 brute force on exactly-summable data, row/column-sum invariants
   masked_add             the reference's smoke vector [1, 1.06, 1, 1.12]
   adamw_masked_decay     step-1 closed forms, torch.optim.AdamW over several steps
+  adamw_step_update      torch.optim.AdamW (amsgrad on/off) in phase 1, phase 1 at eps = 0 in phase 2, step-1 closed forms of Z
   gelu_glu_forward/_backward  torch's gelu(approximate='tanh') * x and autograd's gradient of it
   spmm_ref               dense masked fp32 product (definition); parity of the reference's CUTLASS
                          GEMM itself is unpinned (CUTLASS is an un-vendored, unpinned submodule)
@@ -30,5 +31,6 @@ from .transposable import (  # noqa: F401
 )
 from .decay import masked_add  # noqa: F401
 from .adamw import adamw_masked_decay  # noqa: F401
+from .adamw_step import adamw_step_update, variance_change_statistic  # noqa: F401
 from .gelu_glu import gelu_glu_forward, gelu_glu_backward  # noqa: F401
 from .spmm import spmm_ref, spmm_ref_int, linear_ref  # noqa: F401

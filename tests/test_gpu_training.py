@@ -300,3 +300,92 @@ def test_gelu_glu_errors(cuda):
         sparse.gelu_glu.apply(torch.zeros(2, 3, 4))                       # not on the GPU
     with pytest.raises(AssertionError):
         sparse.gelu_glu.apply(torch.zeros(6, 4, device=cuda))             # the reference asserts a 3-d input
+
+
+@pytest.mark.parametrize("grad_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("amsgrad", [False, True])
+@pytest.mark.parametrize("n,offset", [(4096, 0), (1031, 0), (2050, 1)])
+def test_adamw_step_kernel_matches_oracle(cuda, grad_dtype, amsgrad, n, offset):
+    """tf24_adamw_step against the oracle over several steps, both phases, with the variance-change
+    partial sums; `offset` shifts the tensors off 16-byte alignment (scalar-access variant).
+    Tolerance 2e-6 relative: float32 arithmetic, torch may contract the oracle's multiply-adds."""
+    from sparse import _native as N
+    lib = N.lib()
+    g = torch.Generator().manual_seed(61)
+    hp = dict(lr=2e-3, betas=(0.9, 0.98), eps=1e-7, weight_decay=0.02)
+
+    def dev(t):                                   # a view that starts `offset` elements into its buffer
+        buf = torch.zeros(t.numel() + 8, dtype=t.dtype, device=cuda)
+        buf[offset:offset + t.numel()] = t.to(cuda)
+        return buf[offset:offset + t.numel()]
+
+    p = torch.randn(n, generator=g)
+    m, v = torch.zeros(n), torch.zeros(n)
+    vmax = torch.zeros(n) if amsgrad else None
+    dp, dm, dv = dev(p), dev(m), dev(v)
+    dx = dev(vmax) if amsgrad else None
+    nz = lib.tf24_adamw_step_partials(n)
+    assert nz == (n + 1023) // 1024
+    frozen = None
+    for step in range(1, 6):
+        grad = (torch.randn(n, generator=g) * (1.5 if step % 2 else 0.3)).to(grad_dtype)
+        dg = dev(grad)
+        phase2 = step >= 4
+        if phase2 and frozen is None:
+            frozen = (vmax if amsgrad else v).clone()
+            dfrozen = dev(frozen)
+        for option in ([2, 1] if step == 2 else [1]):       # option 2 runs on copies first: the update itself is the same
+            z = torch.full((nz,), float("nan"), dtype=torch.float32, device=cuda)
+            args = [t.clone() for t in (dp, dm, dv)] if option == 2 else [dp, dm, dv]
+            N.check(lib.tf24_adamw_step(
+                args[0].data_ptr(), dg.data_ptr(), N.dtype_code(grad_dtype), args[1].data_ptr(), args[2].data_ptr(),
+                (dx.clone() if option == 2 else dx).data_ptr() if amsgrad else None, dfrozen.data_ptr() if phase2 else None,
+                n, hp["lr"], hp["betas"][0], hp["betas"][1], hp["eps"], hp["weight_decay"], step,
+                None if phase2 else z.data_ptr(), 0 if phase2 else option, N.stream_ptr()))
+            if not phase2:
+                _, _, _, _, change = oracle.adamw_step_update(p, grad, m, v, step, max_exp_avg_sq=vmax, **hp)
+                want_z = oracle.variance_change_statistic([change], option=option)
+                got = z.double().sum().item() / n
+                got = got if option == 1 else torch.exp(torch.tensor(got, dtype=torch.float64)).item()
+                assert abs(got - want_z) <= 2e-5 * abs(want_z) + 1e-12, (step, option, got, want_z)
+        p, m, v, vmax, _ = oracle.adamw_step_update(p, grad, m, v, step, max_exp_avg_sq=vmax,
+                                                    precond_variance=frozen if phase2 else None, **hp)
+        for got, want in ((dp, p), (dm, m), (dv, v)) + (((dx, vmax),) if amsgrad else ()):
+            assert torch.allclose(got.cpu(), want, rtol=2e-6, atol=1e-9), step
+
+
+def test_adamw_step_optimizer_phases(cuda):
+    """The AdamW_STEP class: watches only parameters carrying `mask`, switches at t > T_max, freezes the
+    variance, and from then on divides tracked parameters by it; untracked ones stay on AdamW."""
+    import sparse
+    torch.manual_seed(62)
+    w = torch.nn.Parameter(torch.randn(48, 40, device=cuda))
+    b = torch.nn.Parameter(torch.randn(40, device=cuda))
+    w.mask = 'dense'
+    hp = dict(lr=1e-2, betas=(0.9, 0.5), eps=1e-8, weight_decay=0.01)
+    opt = sparse.AdamW_STEP([w, b], clipping=(1, 3), option=1, **hp)
+    assert opt.T_omega == 2 and opt.mask == 'dense'
+    ow, ob = w.detach().cpu().clone(), b.detach().cpu().clone()
+    mw, vw, mb, vb = torch.zeros_like(ow), torch.zeros_like(ow), torch.zeros_like(ob), torch.zeros_like(ob)
+    frozen = None
+    g = torch.Generator().manual_seed(63)
+    for t in range(1, 7):
+        gw, gb = torch.randn(48, 40, generator=g), torch.randn(40, generator=g)
+        w.grad, b.grad = gw.to(cuda), gb.to(cuda)
+        opt.step()
+        ow, mw, vw, _, change = oracle.adamw_step_update(ow, gw, mw, vw, t, precond_variance=frozen, **hp)
+        ob, mb, vb, _, _ = oracle.adamw_step_update(ob, gb, mb, vb, t, **hp)
+        assert torch.allclose(w.detach().cpu(), ow, rtol=3e-6, atol=1e-8), t
+        assert torch.allclose(b.detach().cpu(), ob, rtol=3e-6, atol=1e-8), t
+        if t <= 3:
+            assert opt.mask == 'dense' and w.mask == 'dense' and len(opt.sliding_window) == min(t, 2)
+            z = oracle.variance_change_statistic([change], option=1)
+            assert abs(opt.sliding_window[-1].item() - z) <= 1e-5 * z
+        elif t == 4:                                                      # t > T_max = 3: switched after this update
+            assert opt.mask == 'sparse' and w.mask == 'sparse'
+            frozen = vw.clone()
+            assert torch.allclose(opt.state[w]['preconditioned_variance'].cpu(), frozen, rtol=3e-6, atol=1e-12)
+            assert 'preconditioned_variance' not in opt.state[b]
+    assert opt.t == 6 and len(opt.sliding_window) == 2                    # the window stops growing after the switch
+    with pytest.raises(ValueError):
+        sparse.AdamW_STEP([w], option=3)

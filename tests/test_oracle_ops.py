@@ -1,6 +1,7 @@
 """Pins the oracle's MVUE24, soft-threshold, transposable-search and masked-decay functions
 against closed forms, invariants, brute force and the reference's own vectors (CPU only)."""
 import hashlib
+import math
 import os
 import re
 
@@ -241,3 +242,48 @@ def test_gelu_glu_oracle_matches_torch_gelu_and_autograd():
     assert torch.allclose(oracle.gelu_glu_backward(torch.ones(1, 1, 2, dtype=torch.float64), z)[..., 2:], torch.tensor([1.0, -1.5], dtype=torch.float64))
     big = torch.tensor([[[2.0, -3.0, 30.0, -30.0]]], dtype=torch.float64)
     assert torch.allclose(oracle.gelu_glu_forward(big), torch.tensor([[[60.0, 0.0]]], dtype=torch.float64), atol=1e-9)
+
+
+@pytest.mark.parametrize("amsgrad", [False, True])
+def test_adamw_step_oracle_phase1_is_adamw(amsgrad):
+    """Phase 1 of the STEP update is AdamW: compare with torch.optim.AdamW over several steps."""
+    g = torch.Generator().manual_seed(51)
+    p0 = torch.randn(37, 5, generator=g)
+    ref_p = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([ref_p], lr=3e-3, betas=(0.8, 0.95), eps=1e-6, weight_decay=0.05, amsgrad=amsgrad)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    vmax = torch.zeros_like(p0) if amsgrad else None
+    for step in range(1, 7):
+        grad = torch.randn(37, 5, generator=g) * (0.5 if step % 2 else 2.0)      # shrinking gradients exercise the running max
+        ref_p.grad = grad.clone()
+        opt.step()
+        p, m, v, vmax, change = oracle.adamw_step_update(p, grad, m, v, step, lr=3e-3, betas=(0.8, 0.95), eps=1e-6,
+                                                         weight_decay=0.05, max_exp_avg_sq=vmax)
+        assert torch.allclose(p, ref_p.detach(), rtol=2e-6, atol=1e-7)
+    assert (vmax is None) == (not amsgrad)
+
+
+def test_adamw_step_oracle_phase2_and_statistic():
+    g = torch.Generator().manual_seed(52)
+    p0, grad = torch.randn(64, generator=g), torch.randn(64, generator=g)
+    m0, v0 = torch.randn(64, generator=g) * 0.1, torch.rand(64, generator=g) + 0.1
+    kw = dict(lr=1e-2, betas=(0.9, 0.99), eps=0.0, weight_decay=0.01)
+    step = 5
+    p1, m1, v1, _, change = oracle.adamw_step_update(p0, grad, m0, v0, step, **kw)
+    bc2 = 1 - 0.99 ** step
+    # with eps = 0 and the frozen variance v_t / bc2, phase 2 gives phase 1's update
+    p2, m2, v2, _, _ = oracle.adamw_step_update(p0, grad, m0, v0, step, precond_variance=v1 / bc2, **kw)
+    assert torch.allclose(p2, p1, rtol=1e-6, atol=1e-7) and m2.equal(m1) and v2.equal(v1)
+    # with eps > 0 phase 2 adds eps^(3/4) to sqrt(frozen variance), not eps
+    kw["eps"] = 1e-4
+    frozen = torch.full((64,), 4.0)
+    p3, m3, _, _, _ = oracle.adamw_step_update(p0, grad, m0, v0, step, precond_variance=frozen, **kw)
+    want = p0 * (1 - 1e-2 * 0.01) - 1e-2 / (1 - 0.9 ** step) * m3 / (2.0 + 1e-3)
+    assert torch.allclose(p3, want, rtol=1e-6, atol=1e-7)
+    # statistic at step 1 from zero state: v_1 - v_0 = (1 - beta2) g^2
+    _, _, _, _, c1 = oracle.adamw_step_update(p0, grad, torch.zeros(64), torch.zeros(64), 1, **kw)
+    z1 = oracle.variance_change_statistic([c1[:40], c1[40:]], option=1)
+    assert abs(z1 - 0.01 * (grad.double() ** 2).mean().item()) < 1e-6 * z1 + 1e-12
+    z2 = oracle.variance_change_statistic([c1], option=2)
+    assert abs(z2 - 0.01 * math.exp((grad.double() ** 2).log().mean().item())) < 1e-5 * z2
+    assert oracle.variance_change_statistic([torch.zeros(4)], option=2) == 0.0
