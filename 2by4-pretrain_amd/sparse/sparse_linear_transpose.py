@@ -13,9 +13,8 @@ step, mask, weight_sparse, weight_sparse_T, mode.
 import torch
 import torch.nn.functional as F
 from torch import autograd, nn
-from torch.amp import custom_bwd, custom_fwd
 
-from .semi_structured import (SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair,
+from .semi_structured import (SparseSemiStructuredTensor, _spmm, to_sparse_semi_structured, to_sparse_semi_structured_pair,
                               to_sparse_semi_structured_with_row_sums)
 from .transposable_semi_structured import TransposableSparse
 
@@ -23,38 +22,52 @@ __all__ = ["SparseLinearTranspose", "sparse_linear_transpose"]
 
 
 class sparse_linear_transpose(autograd.Function):
-    @staticmethod
-    @custom_fwd(device_type="cuda", cast_inputs=torch.float16)
-    def forward(ctx, input, weight, weight_sparse, weight_sparse_T, bias):
-        ctx.save_for_backward(input, weight_sparse_T, bias)
-        ctx.shape = input.shape
-        input = input.view(-1, input.shape[-1])
-        if bias is None:
-            output = torch.mm(input, weight_sparse.t())
-        else:
-            output = torch.addmm(bias, input, weight_sparse.t())      # bias added in the matmul epilogue
-        return output.view(*ctx.shape[:-1], -1)
+    """README.md:168-200.  The reference decorates forward with custom_fwd(cast_inputs=torch.float16): the
+    arguments are cast and both passes run with autocast off.  That also casts the float32 master
+    `weight` on every call although forward only uses its compressed copies; here the activations
+    and the bias are cast to the compressed copies' dtype and `weight` is left alone.  dW leaves the
+    matmul in the master weight's dtype instead of float16 followed by autograd's cast."""
 
     @staticmethod
-    @custom_bwd(device_type="cuda")
+    def forward(ctx, input, weight, weight_sparse, weight_sparse_T, bias):
+        with torch.autocast(device_type="cuda", enabled=False):
+            compute = weight_sparse.dtype
+            if input.dtype != compute:
+                input = input.to(compute)
+            if bias is not None and bias.dtype != compute:
+                bias = bias.to(compute)
+            ctx.save_for_backward(input, weight_sparse_T, bias)
+            ctx.shape = input.shape
+            ctx.weight_dtype = weight.dtype
+            input = input.view(-1, input.shape[-1])
+            if bias is None:
+                output = torch.mm(input, weight_sparse.t())
+            else:
+                output = torch.addmm(bias, input, weight_sparse.t())      # bias added in the matmul epilogue
+            return output.view(*ctx.shape[:-1], -1)
+
+    @staticmethod
     def backward(ctx, grad_output):
         input, weight_T, bias = ctx.saved_tensors
         grad_input = grad_weight = grad_bias = None
-        if grad_output.stride() == (0,) * grad_output.dim():       # expanded scalar gradient
-            grad_output = torch.ones_like(grad_output)
-        grad_output = grad_output.reshape(-1, grad_output.shape[-1])
-        if ctx.needs_input_grad[0]:
-            grad_input = torch.mm(grad_output, weight_T.t()).view(ctx.shape)
-        if ctx.needs_input_grad[1]:
-            input = input.view(-1, input.shape[-1])
-            if ctx.needs_input_grad[4]:
-                # MVUE24(dY^T) and grad_bias = dY.sum(0) (README.md:193-197) from one read of dY
-                grad_sparse, grad_bias = to_sparse_semi_structured_with_row_sums(grad_output.t(), MVUE24=True, dtype=grad_output.dtype)
-            else:
-                grad_sparse = to_sparse_semi_structured(grad_output.t(), MVUE24=True, dtype=grad_output.dtype)
-            grad_weight = torch.mm(grad_sparse, input)
-        elif ctx.needs_input_grad[4]:
-            grad_bias = grad_output.sum(0)
+        with torch.autocast(device_type="cuda", enabled=False):
+            if grad_output.stride() == (0,) * grad_output.dim():       # expanded scalar gradient
+                grad_output = torch.ones_like(grad_output)
+            grad_output = grad_output.reshape(-1, grad_output.shape[-1])
+            if grad_output.dtype != input.dtype:
+                grad_output = grad_output.to(input.dtype)
+            if ctx.needs_input_grad[0]:
+                grad_input = torch.mm(grad_output, weight_T.t()).view(ctx.shape)
+            if ctx.needs_input_grad[1]:
+                input = input.view(-1, input.shape[-1])
+                if ctx.needs_input_grad[4]:
+                    # MVUE24(dY^T) and grad_bias = dY.sum(0) (README.md:193-197) from one read of dY
+                    grad_sparse, grad_bias = to_sparse_semi_structured_with_row_sums(grad_output.t(), MVUE24=True, dtype=grad_output.dtype)
+                else:
+                    grad_sparse = to_sparse_semi_structured(grad_output.t(), MVUE24=True, dtype=grad_output.dtype)
+                grad_weight = _spmm(grad_sparse, input, True, out_dtype=ctx.weight_dtype)
+            elif ctx.needs_input_grad[4]:
+                grad_bias = grad_output.sum(0)
         return grad_input, grad_weight, None, None, grad_bias
 
 
