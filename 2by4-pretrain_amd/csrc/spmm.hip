@@ -226,7 +226,8 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 // contiguous range of tiles in an 8-tile-high grouped raster: the ~32 tiles resident on an XCD
 // form an 8 x 4 patch that shares A rows and B columns in that XCD's L2.
 // At sustained clocks this kernel runs against the board's power limit (the shader clock settles
-// near 2.1 GHz of 2.4): what buys time is fewer bytes moved per instruction, not a tighter schedule.
+// well below its 2.4 GHz maximum, the lower the more the operand bits toggle): what buys time is
+// fewer bytes moved per instruction, not a tighter schedule.
 // ------------------------------------------------------------------------------------------
 template <typename T> struct mma32;
 template <> struct mma32<f16_t> {
