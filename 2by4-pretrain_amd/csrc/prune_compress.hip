@@ -54,9 +54,8 @@ template <typename In, typename Out, int MODE, typename MaskT>
 __global__ void __launch_bounds__(kThreads)
 prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
-                   const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift,
-                   bool rand_packed) {
+                   RandSrc rs,
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift) {
   constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
   const int64_t upr = k >> 3;                             // 8-element units per row
   const int64_t total = m * upr;
@@ -93,12 +92,15 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       float r[4] = {0.f, 0.f, 0.f, 0.f};
       if constexpr (MODE == TF24_PRUNE_MASK) mk.load_stream(mask + row * mask_ld + col8 * 8);
       if constexpr (MODE == TF24_PRUNE_MVUE) {
-        if (rand_packed) {                                     // [m, k/2]: the unit's four uniforms are adjacent
+        if (rs.kind == RAND_SEEDED) {
+          const Philox4 c = philox4x32_10(rs.seed, (uint64_t)(row * upr + col8), rs.offset);
+          r[0] = philox_uniform(c.x); r[1] = philox_uniform(c.y); r[2] = philox_uniform(c.z); r[3] = philox_uniform(c.w);
+        } else if (rs.kind == RAND_PACKED) {                   // [m, k/2]: the unit's four uniforms are adjacent
           Pack<float, 4> r4;
-          r4.load_stream(rnd + row * rand_ld + col8 * 4);
+          r4.load_stream(rs.ptr + row * rs.ld + col8 * 4);
           r[0] = r4.v[0]; r[1] = r4.v[1]; r[2] = r4.v[2]; r[3] = r4.v[3];
         } else {
-          const float* rp = rnd + row * rand_ld + col8 * 8;
+          const float* rp = rs.ptr + row * rs.ld + col8 * 8;
           Pack<float, 2> ra, rb;                               // the group's two uniforms; read once
           ra.load_stream(rp);
           rb.load_stream(rp + 4);
@@ -134,8 +136,8 @@ template <typename In, typename Out, int MODE, typename MaskT>
 __global__ void __launch_bounds__(kThreads)
 prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
                    const MaskT* __restrict__ mask, int64_t mask_ld,
-                   const float* __restrict__ rnd, int64_t rand_ld,
-                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel, bool rand_packed,
+                   RandSrc rs,
+                   Out* __restrict__ values, uint8_t* __restrict__ meta, bool panel,
                    float* __restrict__ rowsum_partial) {
   constexpr int R = 16 / sizeof(In);
   constexpr int TR = 8 * R;          // tile rows
@@ -158,6 +160,25 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
   float psum[R];
 #pragma unroll
   for (int i = 0; i < R; i++) psum[i] = 0.0f;
+  // Seeded uniforms: one generator call serves the two groups of an 8-column unit, which two lanes
+  // 8 apart own (grp and grp ^ 1).  Each computes the calls of half of the R rows (the even group's
+  // lane the first half) and hands the other lane its two words; every lane of the wave takes part.
+  Pack<float, R> su[2];
+  if constexpr (MODE == TF24_PRUNE_MVUE) {
+    if (rs.kind == RAND_SEEDED) {
+      const int par = grp & 1;
+#pragma unroll
+      for (int j = 0; j < R / 2; j++) {
+        const int64_t row = r0 + j + par * (R / 2);
+        const Philox4 c = philox4x32_10(rs.seed, (uint64_t)(row * (k >> 3) + (c0 >> 3)), rs.offset);
+        const float own0 = philox_uniform(par ? c.z : c.x), own1 = philox_uniform(par ? c.w : c.y);
+        const float snd0 = philox_uniform(par ? c.x : c.z), snd1 = philox_uniform(par ? c.y : c.w);
+        const float rcv0 = __shfl_xor(snd0, 8), rcv1 = __shfl_xor(snd1, 8);
+        su[0].v[j] = par ? rcv0 : own0;          su[1].v[j] = par ? rcv1 : own1;            // row j
+        su[0].v[j + R / 2] = par ? own0 : rcv0;  su[1].v[j + R / 2] = par ? own1 : rcv1;    // row j + R/2
+      }
+    }
+  }
   if (r0 < m && c0 < k) {
     Pack<In, R> in[4];
     Pack<MaskT, R> mk[4];
@@ -169,9 +190,13 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       for (int c = 0; c < 4; c++) mk[c].load_stream(mask + (c0 + c) * mask_ld + r0);
     }
     if constexpr (MODE == TF24_PRUNE_MVUE) {
-      const int64_t rc = rand_packed ? c0 >> 1 : c0;           // packed: columns 2g, 2g+1 of a [m, k/2] tensor
-      rr[0].load_stream(rnd + (rc + 0) * rand_ld + r0);
-      rr[1].load_stream(rnd + (rc + 1) * rand_ld + r0);
+      if (rs.kind == RAND_SEEDED) {
+        rr[0] = su[0]; rr[1] = su[1];
+      } else {
+        const int64_t rc = rs.kind == RAND_PACKED ? c0 >> 1 : c0;   // packed: columns 2g, 2g+1 of a [m, k/2] tensor
+        rr[0].load_stream(rs.ptr + (rc + 0) * rs.ld + r0);
+        rr[1].load_stream(rs.ptr + (rc + 1) * rs.ld + r0);
+      }
     }
 #pragma unroll
     for (int i = 0; i < R; i++) {
@@ -280,10 +305,10 @@ rowsum_finish(const float* __restrict__ partial, int nblocks, int64_t m, T* __re
 
 template <typename In, typename Out, int MODE, typename MaskT>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
-           const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t stream) {
+           RandSrc rs, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t stream) {
   if (layout == TF24_ROW_MAJOR) {
     const int64_t per_block = kThreads * kUnroll;
-    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rand_ld == (rand_packed ? k / 2 : k));
+    const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rs.kind == RAND_SEEDED || rs.ld == (rs.kind == RAND_PACKED ? k / 2 : k));
     const int64_t total = m * (k >> 3);
     dim3 grid((unsigned)((total + per_block - 1) / per_block));
     // lanes per row (log2): 16 lanes read 256 consecutive bytes of bf16 and the four rows of a wave
@@ -294,13 +319,13 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
       grid = dim3((unsigned)(((k >> 3) + units_per_block - 1) / units_per_block), (unsigned)(m / rows_per_block));
     }
     hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
-                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta,
-                       contiguous, panel, lpr_shift, rand_packed);
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rs, (Out*)values, (uint8_t*)meta,
+                       contiguous, panel, lpr_shift);
   } else {
     constexpr int R = 16 / sizeof(In);
     dim3 grid((unsigned)((m + 8 * R - 1) / (8 * R)), (unsigned)((k + 127) / 128));
     hipLaunchKernelGGL((prune_compress_col<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
-                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rnd, rand_ld, (Out*)values, (uint8_t*)meta, panel, rand_packed,
+                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rs, (Out*)values, (uint8_t*)meta, panel,
                        rowsum_partial);
   }
   return check_launch("tf24_prune_compress");
@@ -308,19 +333,19 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
 
 template <typename In, typename Out, int MODE>
 int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int mask_dtype,
-                  int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
+                  int64_t mask_ld, RandSrc rs, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
   if constexpr (MODE != TF24_PRUNE_MASK) {
-    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, nullptr, 0, rs, values, meta, panel, rowsum_partial, s);
   } else if constexpr (std::is_same<In, i8_t>::value) {
     // int8 matrices take byte masks only (the column kernel reads 16 rows per lane: 16-byte mask loads)
     if (mask_dtype != TF24_U8) return fail(TF24_ERR_DTYPE, "tf24_prune_compress: int8 input takes a byte mask (dtype %d given)", mask_dtype);
-    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rs, values, meta, panel, rowsum_partial, s);
   } else {
     switch (mask_dtype) {
-      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      case TF24_U8: return launch<In, Out, MODE, uint8_t>(dense, layout, ld, m, k, mask, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+      case TF24_F16: return launch<In, Out, MODE, f16_t>(dense, layout, ld, m, k, mask, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+      case TF24_BF16: return launch<In, Out, MODE, bf16_t>(dense, layout, ld, m, k, mask, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+      case TF24_F32: return launch<In, Out, MODE, float>(dense, layout, ld, m, k, mask, mask_ld, rs, values, meta, panel, rowsum_partial, s);
     }
     return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported mask dtype %d", mask_dtype);
   }
@@ -328,28 +353,29 @@ int dispatch_mask(const void* dense, int layout, int64_t ld, int64_t m, int64_t 
 
 template <typename In, typename Out>
 int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                  int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
+                  int mask_dtype, int64_t mask_ld, RandSrc rs, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
   switch (mode) {
     case TF24_PRUNE_MAGNITUDE:
-      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MAGNITUDE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
     case TF24_PRUNE_MASK:
-      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      return dispatch_mask<In, Out, TF24_PRUNE_MASK>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
     case TF24_PRUNE_MVUE:
     case TF24_PRUNE_MVUE_PACKED:
+    case TF24_PRUNE_MVUE_SEEDED:
       if constexpr (std::is_same<Out, i8_t>::value) break;        // refused by the validator
-      else return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+      else return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
   }
   return fail(TF24_ERR_ARG, "tf24_prune_compress: bad mode %d", mode);
 }
 
 template <typename In>
 int dispatch_out(int out_dtype, int mode, const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask,
-                 int mask_dtype, int64_t mask_ld, const float* rnd, int64_t rand_ld, bool rand_packed, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
+                 int mask_dtype, int64_t mask_ld, RandSrc rs, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t s) {
   switch (out_dtype) {
-    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_F16: return dispatch_mode<In, f16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_BF16: return dispatch_mode<In, bf16_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_E4M3: return dispatch_mode<In, e4m3_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_E5M2: return dispatch_mode<In, e5m2_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_prune_compress: unsupported output dtype %d", out_dtype);
 }
@@ -367,18 +393,22 @@ int run_prune_compress(const char* fn, const void* dense, int in_dtype, int layo
                                         rnd != nullptr, rand_ld, out_dtype);
   if (rc != TF24_OK) return rc;
   if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "%s: null dense/values/meta pointer", fn);
-  if ((rc = check_aligned(fn, 16, {dense, rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
+  if ((rc = check_aligned(fn, 16, {dense, mode == TF24_PRUNE_MVUE_SEEDED ? nullptr : rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
   if ((rc = check_aligned(fn, 8, {meta, mask}))) return rc;
   if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
     return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, out_layout);
   const bool panel = out_layout == TF24_COMPRESSED_PANEL;
-  const bool rand_packed = mode == TF24_PRUNE_MVUE_PACKED;
+  RandSrc rs{rnd, rand_ld, mode == TF24_PRUNE_MVUE_PACKED ? RAND_PACKED : RAND_FULL, 0, 0};
+  if (mode == TF24_PRUNE_MVUE_SEEDED) {          // `rand` points to {seed, offset} in host memory
+    const uint64_t* so = reinterpret_cast<const uint64_t*>(rnd);
+    rs = RandSrc{nullptr, 0, RAND_SEEDED, so[0], so[1]};
+  }
   hipStream_t s = (hipStream_t)stream;
   switch (in_dtype) {
-    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
-    case TF24_I8: return dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rnd, rand_ld, rand_packed, values, meta, panel, rowsum_partial, s);
+    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_I8: return dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
   }
   return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
 }
@@ -428,5 +458,45 @@ extern "C" int tf24_prune_compress_rowsum(const void* dense, int in_dtype, int l
     case TF24_F16: hipLaunchKernelGGL((rowsum_finish<f16_t>), grid, dim3(kThreads), 0, s, (const float*)workspace, nblocks, m, (f16_t*)rowsum); break;
     default: hipLaunchKernelGGL((rowsum_finish<bf16_t>), grid, dim3(kThreads), 0, s, (const float*)workspace, nblocks, m, (bf16_t*)rowsum); break;
   }
+  return check_launch(fn);
+}
+
+namespace tf24 {
+namespace {
+
+// one lane per generator call: the four packed uniforms of an 8-column unit
+__global__ void __launch_bounds__(kThreads)
+mvue_uniforms_kernel(uint64_t seed, uint64_t offset, int64_t m, int64_t upr, bool col_major, float* __restrict__ out, int64_t ld) {
+  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (u >= m * upr) return;
+  const int64_t row = u / upr, unit = u - row * upr;
+  const Philox4 c = philox4x32_10(seed, (uint64_t)u, offset);
+  const float v[4] = {philox_uniform(c.x), philox_uniform(c.y), philox_uniform(c.z), philox_uniform(c.w)};
+  if (col_major) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[(unit * 4 + i) * ld + row] = v[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[row * ld + unit * 4 + i] = v[i];
+  }
+}
+
+}  // namespace
+}  // namespace tf24
+
+extern "C" int tf24_mvue_uniforms(uint64_t seed, uint64_t offset, int64_t m, int64_t k, int layout, float* out, int64_t ld,
+                                  void* stream) {
+  using namespace tf24;
+  const char* fn = "tf24_mvue_uniforms";
+  if (m <= 0 || k <= 0 || k % 8) return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld): k must be a positive multiple of 8", fn, (long long)m, (long long)k);
+  if (layout != TF24_ROW_MAJOR && layout != TF24_COL_MAJOR) return fail(TF24_ERR_ARG, "%s: bad layout %d", fn, layout);
+  if (ld < (layout == TF24_ROW_MAJOR ? k / 2 : m)) return fail(TF24_ERR_STRIDE, "%s: leading dimension %lld too small", fn, (long long)ld);
+  if (!out) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
+  if (int rc = check_aligned(fn, 4, {out})) return rc;
+  const int64_t total = m * (k / 8);
+  if (total > (int64_t)0x7fffffff * kThreads) return fail(TF24_ERR_SHAPE, "%s: matrix too large", fn);
+  dim3 grid((unsigned)((total + kThreads - 1) / kThreads));
+  hipLaunchKernelGGL(mvue_uniforms_kernel, grid, dim3(kThreads), 0, (hipStream_t)stream, seed, offset, m, k / 8,
+                     layout == TF24_COL_MAJOR, out, ld);
   return check_launch(fn);
 }

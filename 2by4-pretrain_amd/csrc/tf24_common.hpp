@@ -226,6 +226,35 @@ __device__ __forceinline__ float div_in_range(float a, float b, float r) {
   return __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
 }
 
+// Counter-based uniforms for MVUE24 when no tensor is supplied: Philox4x32-10 (Salmon et al., the
+// generator of Random123 / cuRAND / torch), key = seed, counter = {index, offset}.  One call gives
+// the four uniforms of two adjacent groups: `index` = row * (k / 8) + (8-column unit of the row),
+// words 0,1 for the even group of the unit and 2,3 for the odd one.
+struct Philox4 { uint32_t x, y, z, w; };
+__host__ __device__ inline Philox4 philox4x32_10(uint64_t seed, uint64_t index, uint64_t offset) {
+  uint32_t c0 = (uint32_t)index, c1 = (uint32_t)(index >> 32), c2 = (uint32_t)offset, c3 = (uint32_t)(offset >> 32);
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+#pragma unroll
+  for (int round = 0; round < 10; round++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c0 = n0; c1 = (uint32_t)p1; c2 = n2; c3 = (uint32_t)p0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return Philox4{c0, c1, c2, c3};
+}
+// 24 random bits -> [0, 1), exact in float32
+__host__ __device__ inline float philox_uniform(uint32_t bits) { return (float)(bits & 0xffffffu) * 5.9604644775390625e-8f; }
+
+// Where MVUE24 takes its uniforms from
+enum { RAND_FULL = 0, RAND_PACKED = 1, RAND_SEEDED = 2 };
+struct RandSrc {
+  const float* ptr;       // RAND_FULL: [m, k] (columns 4g, 4g+1 used); RAND_PACKED: [m, k/2]
+  int64_t ld;
+  int kind;
+  uint64_t seed, offset;  // RAND_SEEDED
+};
+
 // MVUE24 of one group in float32, in the reference's operation order (no contraction): inclusion
 // probabilities p_i and the kept-mask bits.  The kept values are x_i / p_i (mvue_rescale); only
 // the two kept ones need the division.

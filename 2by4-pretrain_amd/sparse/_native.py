@@ -14,7 +14,7 @@ _lib = None
 # enums of tf24.h
 F32, F16, BF16, E4M3, U8, E5M2, I8, I32 = 0, 1, 2, 3, 4, 5, 6, 7
 ROW_MAJOR, COL_MAJOR = 0, 1
-PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE, PRUNE_MVUE_PACKED = 0, 1, 2, 3
+PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE, PRUNE_MVUE_PACKED, PRUNE_MVUE_SEEDED = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
 COMPRESSED_CANONICAL, COMPRESSED_PANEL = 0, 1
 
@@ -34,6 +34,7 @@ _SIGNATURES = {
     "tf24_last_error": (ctypes.c_char_p, []),
     "tf24_prune_compress": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p]),
     "tf24_prune_compress_validate": (_i, [_i, _i, _i64, _i64, _i64, _i, _i, _i, _i64, _i, _i64, _i]),
+    "tf24_mvue_uniforms": (_i, [ctypes.c_uint64, ctypes.c_uint64, _i64, _i64, _i, _p, _i64, _p]),
     "tf24_prune_compress_rowsum": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p, _i, _p, _i64, _p]),
     "tf24_prune_compress_rowsum_workspace_bytes": (_i64, [_i64, _i64]),
     "tf24_prune_compress_dual": (_i, [_p, _i, _i64, _i64, _i64, _p, _i, _i64, _p, _p, _p, _p, _i, _i, _p]),

@@ -11,9 +11,11 @@ behaviour.  Differences, all deliberate:
     (values [m, k/2], nibble metadata [m, k/16 | k/32]) on first use, also for column-major
     inputs (`W.T`); the metadata is the canonical nibble stream, not CUTLASS's reordered layout --
     `indices_cutlass()` exports the reordered form;
-  * MVUE24 takes its uniforms from an optional `rand` tensor (drawn with torch.rand when omitted);
+  * MVUE24 takes its uniforms from an optional `rand` tensor, or generates them inside the kernel from
+    (seed, offset) -- `rand=(seed, offset)`, or torch's generator state when `rand` is omitted;
   * `addmm` / `linear` with a bias work (the reference passes a wrong keyword there).
 """
+import ctypes
 import warnings
 from collections import namedtuple
 from typing import Any, Optional
@@ -62,6 +64,24 @@ def _to_canonical(values, meta, m, n):
     return v, mt
 
 
+class _HostWords:
+    """A ctypes array passed where the binding expects a tensor's data_ptr()."""
+    def __init__(self, array):
+        self.array = array
+
+    def data_ptr(self):
+        return ctypes.addressof(self.array)
+
+
+def _next_philox_state(device):
+    """(seed, offset) of torch's generator for `device`, advancing its offset the way a random op does,
+    so that torch.manual_seed() makes the default MVUE24 sampling reproducible."""
+    gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+    offset = gen.get_offset()
+    gen.set_offset(offset + 4)
+    return gen.initial_seed(), offset
+
+
 def _compress(original, dtype, MVUE24, mask, rand, panel, row_sums=False):
     """One allocation of numel*cf/16 elements: values first, metadata in the tail
     (reference :215-243); then the HIP prune+compress kernel.  Returns flat storage views; with
@@ -96,18 +116,19 @@ def _compress(original, dtype, MVUE24, mask, rand, panel, row_sums=False):
     elif MVUE24:
         mode = N.PRUNE_MVUE
         if rand is None:
-            # only two uniforms per group of four are used: draw [m, n/2] in the dense operand's layout
-            if layout == N.ROW_MAJOR:
-                rand = torch.rand((m, n // 2), dtype=torch.float32, device=dense.device)
-            else:
-                rand = torch.rand((n // 2, m), dtype=torch.float32, device=dense.device).t()
-        if tuple(rand.shape) == (m, n // 2):
-            mode = N.PRUNE_MVUE_PACKED               # group g of a row uses rand[r, 2g], rand[r, 2g+1]
-        elif rand.shape != original.shape:
-            raise RuntimeError(f"rand shape {tuple(rand.shape)} does not match tensor shape {tuple(original.shape)} "
-                               f"(or its packed form {(m, n // 2)})")
-        rand_t = N.as_matrix(rand.float(), like=dense)
-        rand_ld = N.layout_of(rand_t)[1]
+            rand = _next_philox_state(dense.device)  # uniforms generated inside the kernel
+        if isinstance(rand, tuple):
+            mode = N.PRUNE_MVUE_SEEDED
+            seed_offset = (ctypes.c_uint64 * 2)(int(rand[0]) & (2 ** 64 - 1), int(rand[1]) & (2 ** 64 - 1))
+            rand_t = _HostWords(seed_offset)         # read by the library during the call
+        else:
+            if tuple(rand.shape) == (m, n // 2):
+                mode = N.PRUNE_MVUE_PACKED           # group g of a row uses rand[r, 2g], rand[r, 2g+1]
+            elif rand.shape != original.shape:
+                raise RuntimeError(f"rand shape {tuple(rand.shape)} does not match tensor shape {tuple(original.shape)} "
+                                   f"(or its packed form {(m, n // 2)})")
+            rand_t = N.as_matrix(rand.float(), like=dense)
+            rand_ld = N.layout_of(rand_t)[1]
     if row_sums:
         sums = torch.empty((m,), dtype=dense.dtype, device=dense.device)
         ws_bytes = N.lib().tf24_prune_compress_rowsum_workspace_bytes(m, n)
@@ -415,8 +436,9 @@ def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = 
 
     Without `mask`/`MVUE24` the two largest |x| of every 4 are kept (ties: larger index);
     `mask` (same shape, nonzero = keep) selects explicitly; `MVUE24=True` samples the
-    minimum-variance unbiased estimator, taking its uniforms from `rand` (same shape, U[0,1);
-    drawn with torch's generator when omitted).  `dtype` is the value dtype of the result
+    minimum-variance unbiased estimator, taking its uniforms from `rand`: a tensor of the same shape
+    (or the packed [m, k/2] form) in [0,1), or a (seed, offset) pair for uniforms generated inside the
+    kernel; when omitted, the pair is taken from torch's generator (torch.manual_seed applies).  `dtype` is the value dtype of the result
     (float16, bfloat16, float8_e4m3fn, float8_e5m2, or int8 for an int8 tensor).  Rows must be a
     multiple of 32, columns of 64 (128 for 8-bit values).  Same signature as the reference's factory (semi_structured.py:575-631)
     plus `rand`.

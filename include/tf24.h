@@ -54,7 +54,10 @@ typedef enum {
   TF24_PRUNE_MAGNITUDE = 0, /* keep the 2 largest |x| per group, ties -> larger index */
   TF24_PRUNE_MASK = 1,      /* keep what a supplied mask says */
   TF24_PRUNE_MVUE = 2,      /* MVUE24 sampling from a supplied U(0,1) tensor of the dense shape */
-  TF24_PRUNE_MVUE_PACKED = 3 /* the same with only the uniforms that are used: a [m, k/2] tensor */
+  TF24_PRUNE_MVUE_PACKED = 3, /* the same with only the uniforms that are used: a [m, k/2] tensor */
+  TF24_PRUNE_MVUE_SEEDED = 4  /* MVUE24 with uniforms generated in the kernel: `rand` points to two uint64
+                                 values {seed, offset} in HOST memory (read during the call).  The uniforms
+                                 are exactly those tf24_mvue_uniforms writes for the same seed and offset. */
 } tf24_prune_mode;
 
 /* GELU is the exact (erf) form, torch.nn.functional.gelu's default; the reference's epilogues stop at SILU */
@@ -98,6 +101,17 @@ int tf24_prune_compress(const void* dense, int in_dtype, int layout, int64_t ld,
                         int mode, const void* mask, int mask_dtype, int64_t mask_ld,
                         const float* rand, int64_t rand_ld,
                         void* values, int out_dtype, void* meta, int out_layout, void* stream);
+
+/*
+ * The packed uniforms [m, k/2] of TF24_PRUNE_MVUE_SEEDED as a tensor: Philox4x32-10 with key = seed and
+ * counter = {row * (k/8) + c/4, offset} yields columns 4*(c/4) .. 4*(c/4)+3 of row `row`; each word gives
+ * (word & 0xffffff) * 2^-24 in [0, 1).  The reference seeds an in-kernel Philox from Python's `random`
+ * (sparse/_semi_structured_conversions.py:536-542, :1076), which is not reproducible; this one is, from
+ * (seed, offset).  out: float32, TF24_ROW_MAJOR [m, k/2] with leading dimension ld >= k/2, or
+ * TF24_COL_MAJOR (element (r, c) at c*ld + r, ld >= m).  k % 8 == 0.
+ */
+int tf24_mvue_uniforms(uint64_t seed, uint64_t offset, int64_t m, int64_t k, int layout, float* out, int64_t ld,
+                       void* stream);
 
 /*
  * tf24_prune_compress of a column-major matrix that also returns its row sums,

@@ -13,6 +13,7 @@ Pinning status (what fixes each function independently of this file):
   mvue24                 sum(p)=2, analytic inclusion probabilities, Monte-Carlo unbiasedness
   soft_threshold24       closed form (2nd smallest |a|), sort-based restatement on tie-free data
   transposable_mask      90-way fp64 brute force on exactly-summable data, row/column-sum invariants
+  philox4x32_10          Random123's known-answer vectors
   masked_add             the reference's smoke vector [1, 1.06, 1, 1.12]
   adamw_masked_decay     step-1 closed forms, torch.optim.AdamW over several steps
   adamw_step_update      torch.optim.AdamW (amsgrad on/off) in phase 1, phase 1 at eps = 0 in phase 2, step-1 closed forms of Z
@@ -30,6 +31,7 @@ from .transposable import (  # noqa: F401
     transposable_patterns, transposable_mask, transposable_mask_bruteforce,
 )
 from .decay import masked_add  # noqa: F401
+from .philox import philox4x32_10, mvue_uniforms  # noqa: F401
 from .adamw import adamw_masked_decay  # noqa: F401
 from .adamw_step import adamw_step_update, variance_change_statistic  # noqa: F401
 from .gelu_glu import gelu_glu_forward, gelu_glu_backward  # noqa: F401

@@ -299,6 +299,58 @@ def test_mvue_compress_packed_uniforms(cuda, out_dtype, col_major):
         sparse.to_sparse_semi_structured(w.to(cuda), MVUE24=True, rand=up[:, :-8].to(cuda), dtype=out_dtype)
 
 
+@pytest.mark.parametrize("col_major", [False, True])
+@pytest.mark.parametrize("in_dtype,out_dtype,shape", [(BF16, F16, (64, 128)), (F16, F16, (96, 320)), (F32, BF16, (32, 64)), (F16, E4M3, (64, 256))])
+def test_mvue_seeded_uniforms(cuda, in_dtype, out_dtype, shape, col_major):
+    """Uniforms generated inside the kernel: tf24_mvue_uniforms writes the oracle's Philox stream, and
+    compressing with rand=(seed, offset) gives the bytes of compressing with that tensor supplied."""
+    import sparse
+    from sparse import _native as N
+    m, k = shape
+    seed, offset = 0x1234567890abcdef, 40
+    want_u = oracle.mvue_uniforms(seed, offset, m, k)
+    got = torch.empty((m, k // 2), dtype=torch.float32, device=cuda)
+    N.check(N.lib().tf24_mvue_uniforms(seed, offset, m, k, N.ROW_MAJOR, got.data_ptr(), k // 2, N.stream_ptr()))
+    assert got.cpu().equal(want_u)
+    got_t = torch.empty((k // 2, m), dtype=torch.float32, device=cuda)
+    N.check(N.lib().tf24_mvue_uniforms(seed, offset, m, k, N.COL_MAJOR, got_t.data_ptr(), m, N.stream_ptr()))
+    assert got_t.t().cpu().equal(want_u)
+    w = randn(shape, in_dtype, 23)
+    full = torch.zeros(shape)
+    full[:, 0::4], full[:, 1::4] = want_u[:, 0::2], want_u[:, 1::2]
+    want_v, want_m, _ = oracle.mvue24(w, full, out_dtype=out_dtype)
+    wd = maybe_t(w.to(cuda), col_major)
+    s = sparse.to_sparse_semi_structured(wd, MVUE24=True, dtype=out_dtype, rand=(seed, offset))
+    assert_same(s.values(), want_v, "values")
+    assert_same(s.indices(), want_m, "meta")
+    if col_major and out_dtype not in FLOAT8:
+        s2, sums = sparse.to_sparse_semi_structured_with_row_sums(wd, MVUE24=True, dtype=out_dtype, rand=(seed, offset))
+        assert_same(s2.values(), want_v)
+        assert_same(s2.indices(), want_m)
+
+
+def test_mvue_default_sampling_follows_torch_seed(cuda):
+    """Without `rand` the (seed, offset) pair comes from torch's generator: torch.manual_seed makes the
+    sampling reproducible, successive calls draw different uniforms, two values are kept per group."""
+    import sparse
+    w = randn((64, 256), F16, 24).to(cuda)
+    torch.manual_seed(77)
+    a1 = sparse.to_sparse_semi_structured(w, MVUE24=True)
+    a2 = sparse.to_sparse_semi_structured(w, MVUE24=True)
+    torch.manual_seed(77)
+    b1 = sparse.to_sparse_semi_structured(w.t().contiguous().t(), MVUE24=True)      # same matrix, column-major storage
+    assert a1.indices().equal(b1.indices()) and a1.values().equal(b1.values())
+    assert not a1.indices().equal(a2.indices())
+    dense = a1.to_dense()
+    assert ((dense != 0).view(64, 64, 4).sum(-1) <= 2).all()
+    # unbiased: the mean over many draws approaches w
+    acc = torch.zeros_like(w, dtype=torch.float32)
+    for _ in range(200):
+        acc += sparse.to_sparse_semi_structured(w, MVUE24=True).to_dense().float()
+    err = (acc / 200 - w.float()).abs().mean() / w.float().abs().mean()
+    assert err < 0.12, err
+
+
 def _wide_range(shape, seed):
     """float32 values whose exponents span denormals to 2^60, with zeros, negative zeros and groups
     dominated by one element (sum - a_i rounds to zero): operands the in-range division must hand

@@ -287,3 +287,20 @@ def test_adamw_step_oracle_phase2_and_statistic():
     z2 = oracle.variance_change_statistic([c1], option=2)
     assert abs(z2 - 0.01 * math.exp((grad.double() ** 2).log().mean().item())) < 1e-5 * z2
     assert oracle.variance_change_statistic([torch.zeros(4)], option=2) == 0.0
+
+
+def test_philox_known_answers():
+    """Philox4x32-10 against the known-answer vectors of the Random123 distribution."""
+    import numpy as np
+    kats = [([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+            ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+            ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0], [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1])]
+    for counter, key, want in kats:
+        got = oracle.philox4x32_10(np.array(counter, dtype=np.uint64), np.array(key, dtype=np.uint64))
+        assert [int(x) for x in got] == want
+    u = oracle.mvue_uniforms(seed=1234, offset=8, m=32, k=64)
+    assert u.shape == (32, 32) and u.dtype == torch.float32 and (u >= 0).all() and (u < 1).all()
+    assert abs(u.mean().item() - 0.5) < 0.05 and not u.equal(oracle.mvue_uniforms(1234, 12, 32, 64))
+    # row r, unit q of the row uses counter index r * (k/8) + q: the first unit of row 1 is call number k/8
+    words = oracle.philox4x32_10(np.array([8, 0, 8, 0], dtype=np.uint64), np.array([1234, 0], dtype=np.uint64))
+    assert u[1, 0].item() == float(int(words[0]) & 0xffffff) * 2.0 ** -24
