@@ -3,15 +3,16 @@
  * huyz2023/2by4-pretrain, hand-written for MI355X (gfx950 / CDNA4).
  *
  * Conventions
- *   - Every pointer is a DEVICE pointer (HIP) unless the name ends in _host.
+ *   - Every pointer is a DEVICE pointer (HIP); the one exception is `rand` in mode
+ *     TF24_PRUNE_MVUE_SEEDED, which points to {seed, offset} in host memory.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Nothing here
  *     allocates, frees or synchronises: the caller owns every buffer, work is only enqueued.
  *   - Return value: TF24_OK or a negative tf24_status; tf24_last_error() returns a
  *     thread-local human readable message for the last failure on the calling thread.
  *   - A logical [m,k] matrix is described by (layout, ld):
  *       TF24_ROW_MAJOR element (r,c) at r*ld + c,   TF24_COL_MAJOR element (r,c) at c*ld + r.
- *   - "group" = 4 consecutive elements along k.  Compressed values are always written
- *     row-major [m, k/2]; metadata is the canonical nibble stream: for each group
+ *   - "group" = 4 consecutive elements along k.  In the canonical compressed form the values are
+ *     row-major [m, k/2] and the metadata is the nibble stream: for each group
  *     pos0 | pos1<<2 (pos0 < pos1 = positions of the two kept elements), packed LSB-first
  *     into int16 [m, k/16] for 16-bit values or int32 [m, k/32] for 8-bit values.  One int16
  *     is exactly the index operand of one lane of V_SMFMAC_F32_16X16X64_{F16,BF16}; one int32
