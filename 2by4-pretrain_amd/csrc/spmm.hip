@@ -567,13 +567,15 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 #pragma unroll
     for (int ti = 0; ti < C::TI; ti++)
 #pragma unroll
-      for (int tj = 0; tj < C::TJ; tj++)
+      for (int tj = 0; tj < C::TJ; tj++) {
+        if (j0 + wj * C::WJ + tj * 32 >= n_dense) continue;      // columns past the dense operand: never read back
 #pragma unroll
         for (int g = 0; g < 4; g++) {
           const int slab = (ti * C::TJ + tj) * 4 + g;
           typename mma32<T>::acc4_t v = {acc[ti][tj][g * 4], acc[ti][tj][g * 4 + 1], acc[ti][tj][g * 4 + 2], acc[ti][tj][g * 4 + 3]};
           *reinterpret_cast<typename mma32<T>::acc4_t*>(base + ((int64_t)slab * C::THREADS + tid) * 4) = v;
         }
+      }
     return;
   }
 
@@ -704,6 +706,7 @@ spmm_reduce_splits(const float* __restrict__ partial, int splits, int tiles_i, i
   // gridDim.y blocks share the NSLAB accumulator groups of the tile
   for (int slab = blockIdx.y; slab < NSLAB; slab += gridDim.y) {
     const int ti = slab / (C::TJ * 4), tj = (slab / 4) % C::TJ, g = slab % 4;
+    if (j0 + wj * C::WJ + tj * 32 >= n_dense) continue;          // the whole 32-column slab lies past the dense operand
     Acc4 sum = {0, 0, 0, 0};
     for (int sp = 0; sp < splits; sp++) {
       const float* base = partial + ((int64_t)sp * ntiles + tile) * (C::BI * C::BJ);
@@ -796,7 +799,8 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  void* workspace, int64_t workspace_bytes, hipStream_t s) {
   // the tiled kernel reads a k-strided dense operand through transposing LDS reads (16-bit types only)
-  const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64 && n_dense >= 64;
+  // (also for a narrow dense operand: with its k pieces the tiled kernel beats the general one from 8 columns on)
+  const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64;
   if constexpr (std::is_same<T, i8_t>::value) {        // integer product: int32 accumulators, results and bias
     if (tiled) return launch_tiled<T, int32_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     return launch_general<T, int32_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);

@@ -155,7 +155,7 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     n, k = sparse._store_shape
     # An operand built from canonical values/metadata (the functional entry point) is brought to the
     # panel form once: the tiled kernel only streams that one.
-    if (store_layout == N.COMPRESSED_CANONICAL and n >= 64 and dense.numel() // k >= 64 and k % _panel_width(values.dtype) == 0):
+    if store_layout == N.COMPRESSED_CANONICAL and n >= 64 and k % _panel_width(values.dtype) == 0:
         pv, pm = torch.empty_like(values), torch.empty_like(meta)
         N.check(N.lib().tf24_repack(values.data_ptr(), meta.data_ptr(), N.operand_code(values.dtype), n, k, N.COMPRESSED_CANONICAL,
                                     pv.data_ptr(), pm.data_ptr(), N.stream_ptr()))
