@@ -798,3 +798,27 @@ def test_int8_spmm_extreme_values(cuda):
     s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=torch.int8)
     out = torch.mm(x.to(cuda), s.t())
     assert out.cpu().equal(torch.full((m, n), 16384 * (k // 2), dtype=torch.int32))
+
+
+@pytest.mark.parametrize("dtype,m", [(F16, 8), (F16, 24), (BF16, 40), (E4M3, 16), (torch.int8, 16)])
+@pytest.mark.parametrize("k", [512, 4096])
+def test_spmm_narrow_dense_operand(cuda, dtype, m, k):
+    """A handful of dense columns against a tall sparse operand: the tiled kernel (with k pieces at
+    k = 4096) whose partial tiles only cover the live 32-column slabs; every operand position and layout."""
+    import sparse
+    n = 320
+    if dtype == torch.int8:
+        w, x = _int8((n, k), 121, -3, 4), _int8((m, k), 122, -3, 4)
+        ref = oracle.spmm_ref_int(x, torch.where(oracle.prune24_mask(w.float()), w, torch.zeros_like(w)))
+        s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    else:
+        w, x = _small_ints((n, k), 121, -2, 3).to(dtype), _small_ints((m, k), 122, -2, 3).to(dtype)
+        mask = oracle.prune24_mask(w.float())
+        ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+        s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    xg = x.to(cuda)
+    same = lambda out, want: out.cpu().to(torch.float64).equal(want.to(out.dtype).to(torch.float64))
+    assert same(torch.mm(xg, s.t()), ref)
+    assert same(torch.mm(maybe_t(xg, True), s.t()), ref)
+    assert same(torch.mm(s, xg.t()), ref.t())
+    assert same(torch.mm(s, xg.t().contiguous()), ref.t())
