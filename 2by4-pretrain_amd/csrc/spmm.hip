@@ -778,6 +778,99 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   return check_launch("tf24_spmm");
 }
 
+// ------------------------------------------------------------------------------------------
+// Narrow kernel: at most 16 dense columns (decoding a few tokens against a large sparse weight).
+// The product is bound by one pass over the compressed operand, so nothing is staged: a block owns
+// 16 sparse rows; its waves (one when the rows alone give enough blocks to fill the chip, otherwise
+// up to four, each taking a share of the k range) run one V_SMFMAC_*_16X16 per panel and meet in
+// LDS at the end (added in wave order).  In the panel layout the A fragments of
+// 16 adjacent rows are 1 KB of contiguous memory (16 bytes per lane) and their index words 128
+// (256) contiguous bytes; the dense fragment is 64 contiguous bytes from each of the 16 dense rows,
+// twice.  Loads are issued 16 panels at a time (about 16 KB of the sparse operand per wave in
+// flight): left to itself the compiler waits for each panel's loads before it issues the next.
+// ------------------------------------------------------------------------------------------
+constexpr int kNarrowMaxDense = 16;
+constexpr int kNarrowWaves = 4;
+
+template <typename T, typename OutT, bool C_JMAJOR>
+__global__ void __launch_bounds__(64 * kNarrowWaves)
+spmm_narrow(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
+            const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
+            OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
+  constexpr int KSTEP = mma16<T>::KSTEP;     // dense k per panel = per instruction
+  constexpr int M_ROW = KSTEP / 8;           // metadata bytes per row per panel
+  constexpr int BATCH = 16;
+  using acc_t = typename mma16<T>::acc_t;
+  __shared__ acc_t s_acc[kNarrowWaves - 1][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, lk = lane >> 4;
+  const int64_t i0 = (int64_t)blockIdx.x * 16;
+  const int64_t npanels = k / KSTEP;
+  const int nwaves = blockDim.x >> 6;
+  const int64_t p_begin = wave * npanels / nwaves, p_end = (wave + 1) * npanels / nwaves;
+  const int64_t col = li < n_dense ? li : n_dense - 1;          // clamp: the column is never stored
+  const uint8_t* bp = b + col * ldb_bytes + lk * 16;
+  const uint8_t* av = a_values + (i0 + li) * 64 + lk * 16;
+  const uint8_t* am = a_meta + (i0 + li) * M_ROW + lk * (M_ROW / 4);
+  const int64_t a_step = n_sparse * 64, m_step = n_sparse * M_ROW;
+  acc_t acc[2];                              // two chains, so that consecutive instructions do not wait on each other
+#pragma unroll
+  for (int r = 0; r < 4; r++) { acc[0][r] = 0; acc[1][r] = 0; }
+  for (int64_t p = p_begin; p < p_end; p += BATCH) {
+    int4v af[BATCH], lo[BATCH], hi[BATCH];
+    int idx[BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; u++) {
+      const int64_t pp = p + u < p_end ? p + u : p_end - 1;     // past the end: re-read the last panel, multiply by zero
+      af[u] = __builtin_nontemporal_load(reinterpret_cast<const int4v*>(av + pp * a_step));
+      if constexpr (sizeof(T) == 2) idx[u] = *reinterpret_cast<const uint16_t*>(am + pp * m_step);
+      else idx[u] = *reinterpret_cast<const int*>(am + pp * m_step);
+      lo[u] = *reinterpret_cast<const int4v*>(bp + pp * 128);
+      hi[u] = *reinterpret_cast<const int4v*>(bp + pp * 128 + 64);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < BATCH; u++) {
+      if (p + u >= p_end) af[u] = int4v{0, 0, 0, 0};
+      const int8v bfrag = {lo[u][0], lo[u][1], lo[u][2], lo[u][3], hi[u][0], hi[u][1], hi[u][2], hi[u][3]};
+      acc[u & 1] = mma16<T>::template run<0>(af[u], bfrag, acc[u & 1], idx[u]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  acc_t sum = acc[0] + acc[1];
+  if (wave > 0) s_acc[wave - 1][lane] = sum;
+  __syncthreads();
+  if (wave > 0 || li >= n_dense) return;
+#pragma unroll
+  for (int w = 0; w < nwaves - 1; w++) sum += s_acc[w][lane];
+  const int64_t row = i0 + lk * 4;           // D layout: column l%16, rows 4*(l/16) + r
+  OutT o[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_value(sum[r], scale, bias, row + r, act));
+  if constexpr (C_JMAJOR) {
+    *reinterpret_cast<Pack<OutT, 4>*>(c + (int64_t)li * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; r++) c[(row + r) * ldc + li] = o[r];
+  }
+}
+
+template <typename T, typename OutT>
+int launch_narrow(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb, int64_t n_dense,
+                  void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
+  dim3 grid((unsigned)(n_sparse / 16));
+  // waves per block: one 16-row block per wave when that already gives two waves per CU, else split k
+  const int64_t blocks = n_sparse / 16, npanels = k * (int64_t)sizeof(T) / 128;
+  int nwaves = blocks >= 512 ? 1 : kNarrowWaves;
+  while (nwaves > 1 && npanels / nwaves < 4) nwaves /= 2;
+  if (c_layout == TF24_COL_MAJOR)
+    hipLaunchKernelGGL((spmm_narrow<T, OutT, true>), grid, dim3(64 * nwaves), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
+                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
+  else
+    hipLaunchKernelGGL((spmm_narrow<T, OutT, false>), grid, dim3(64 * nwaves), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
+                       (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
+  return check_launch("tf24_spmm");
+}
+
 template <typename T, typename OutT>
 int launch_general(const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                    int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
@@ -801,10 +894,20 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
   // the tiled kernel reads a k-strided dense operand through transposing LDS reads (16-bit types only)
   // (also for a narrow dense operand: with its k pieces the tiled kernel beats the general one from 8 columns on)
   const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64;
+  // at most 16 dense columns: one pass over the compressed operand, no staging
+  const bool narrow = panel && b_layout == TF24_ROW_MAJOR && n_dense <= kNarrowMaxDense;
   if constexpr (std::is_same<T, i8_t>::value) {        // integer product: int32 accumulators, results and bias
+    if (narrow) return launch_narrow<T, int32_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
     if (tiled) return launch_tiled<T, int32_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     return launch_general<T, int32_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   } else {
+  if (narrow) {
+    switch (out_dtype) {
+      case TF24_F16: return launch_narrow<T, f16_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_BF16: return launch_narrow<T, bf16_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+      case TF24_F32: return launch_narrow<T, float>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    }
+  }
   if (tiled) {
     switch (out_dtype) {
       case TF24_F16: return launch_tiled<T, f16_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);

@@ -822,3 +822,24 @@ def test_spmm_narrow_dense_operand(cuda, dtype, m, k):
     assert same(torch.mm(maybe_t(xg, True), s.t()), ref)
     assert same(torch.mm(s, xg.t()), ref.t())
     assert same(torch.mm(s, xg.t().contiguous()), ref.t())
+
+
+@pytest.mark.parametrize("dtype", [F16, E4M3])
+def test_spmm_narrow_one_wave_per_block(cuda, dtype):
+    """Many sparse rows and at most 16 dense columns: the narrow kernel runs one wave per 16-row block
+    (fewer rows split k over four waves: test_spmm_narrow_dense_operand); k not a multiple of its
+    16-panel load batch."""
+    import sparse
+    n, k, m = 8192, 1408 if dtype == F16 else 2816, 16
+    w, x = _small_ints((n, k), 131, -2, 3).to(dtype), _small_ints((m, k), 132, -2, 3).to(dtype)
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    bias = _small_ints((n,), 133).to(torch.float32 if dtype == E4M3 else dtype)
+    out = torch.mm(x.to(cuda), s.t())
+    assert out.float().cpu().equal(ref.to(out.dtype).float())
+    out = torch.mm(s, x.to(cuda).t())
+    assert out.float().cpu().equal(ref.t().to(out.dtype).float())
+    out = sparse.sparse_semi_structured_linear(x.to(cuda)[:8], s, bias=bias.to(cuda), activation="relu")
+    want = (ref[:8] + bias.float()).clamp_min(0)
+    assert out.float().cpu().equal(want.to(out.dtype).float())
