@@ -275,7 +275,7 @@ struct TileCfgT {
   static constexpr int TI = 4, TJ = TJ_;         // 32x32 instructions per wave
   static constexpr int WI = 32 * TI, WJ = 32 * TJ;
   static constexpr int BI = WI * WAVES_I, BJ = WJ * WAVES_J;
-  static_assert(BI == 256 && BJ == 256, "stage buffers are sized for 256 x 256 tiles");
+  static_assert(BI == 256 && (BJ == 256 || BJ == 64), "stage buffers are sized for 256 x 256 and 256 x 64 tiles");
   static constexpr int KB = 128;                 // bytes of dense k per row per stage
   static constexpr int STEPS = KB / 64;          // instruction steps per stage
   static constexpr int A_ROW = KB / 2;           // LDS bytes per row per stage: compressed values
@@ -285,6 +285,9 @@ struct TileCfgT {
   static constexpr int NA = BI * A_ROW / 1024 / NW;   //                                 A values
 };
 using TiledCfg = TileCfgT<4, 2>;
+// 256 x 64 tiles, two waves: for dense operands of at most 64 columns (a few dozen tokens), where a
+// 256-wide tile would copy and multiply clamped columns.  26 KB per stage, two blocks per CU.
+using SlimCfg = TileCfgT<1, 2>;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -756,9 +759,9 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
                        (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
   };
   bool kstrided = false;
-  if constexpr (sizeof(T) == 2) kstrided = b_layout == TF24_COL_MAJOR;
+  if constexpr (sizeof(T) == 2 && C::BJ == 256) kstrided = b_layout == TF24_COL_MAJOR;
   if (kstrided) {
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (sizeof(T) == 2 && C::BJ == 256) {
       if (jm) launch(std::true_type{}, std::true_type{});
       else launch(std::false_type{}, std::true_type{});
     }
@@ -896,8 +899,11 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
   const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64;
   // at most 16 dense columns: one pass over the compressed operand, no staging
   const bool narrow = panel && b_layout == TF24_ROW_MAJOR && n_dense <= kNarrowMaxDense;
+  // up to 64 dense columns: the tiled kernel on 256 x 64 tiles
+  const bool slim = tiled && b_layout == TF24_ROW_MAJOR && n_dense <= SlimCfg::BJ;
   if constexpr (std::is_same<T, i8_t>::value) {        // integer product: int32 accumulators, results and bias
     if (narrow) return launch_narrow<T, int32_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    if (slim) return launch_tiled<T, int32_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     if (tiled) return launch_tiled<T, int32_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     return launch_general<T, int32_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   } else {
@@ -906,6 +912,13 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
       case TF24_F16: return launch_narrow<T, f16_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
       case TF24_BF16: return launch_narrow<T, bf16_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
       case TF24_F32: return launch_narrow<T, float>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    }
+  }
+  if (slim) {
+    switch (out_dtype) {
+      case TF24_F16: return launch_tiled<T, f16_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_BF16: return launch_tiled<T, bf16_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_F32: return launch_tiled<T, float, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     }
   }
   if (tiled) {
@@ -960,9 +973,17 @@ extern "C" int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_
   int splits;
   if (is_8bit(dtype)) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
   else splits = choose_splits<f16_t, TiledCfg>(n_sparse, k, n_dense, big);
-  if (splits < 2) return 0;
-  const int64_t tiles = ((n_sparse + TiledCfg::BI - 1) / TiledCfg::BI) * ((n_dense + TiledCfg::BJ - 1) / TiledCfg::BJ);
-  return splits * tiles * TiledCfg::BI * TiledCfg::BJ * 4;
+  int64_t bytes = 0;
+  if (splits >= 2) {
+    const int64_t tiles = ((n_sparse + TiledCfg::BI - 1) / TiledCfg::BI) * ((n_dense + TiledCfg::BJ - 1) / TiledCfg::BJ);
+    bytes = splits * tiles * TiledCfg::BI * TiledCfg::BJ * 4;
+  }
+  if (n_dense <= SlimCfg::BJ) {              // the 64-wide tile's k pieces
+    const int ss = is_8bit(dtype) ? choose_splits<e4m3_t, SlimCfg>(n_sparse, k, n_dense, big) : choose_splits<f16_t, SlimCfg>(n_sparse, k, n_dense, big);
+    const int64_t need = ss >= 2 ? (int64_t)ss * ((n_sparse + SlimCfg::BI - 1) / SlimCfg::BI) * SlimCfg::BI * SlimCfg::BJ * 4 : 0;
+    if (need > bytes) bytes = need;
+  }
+  return bytes;
 }
 
 extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,

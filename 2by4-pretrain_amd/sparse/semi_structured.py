@@ -170,8 +170,8 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     # loads fragments.  For 8-bit operands it wants k contiguous: one transposing copy of the dense
     # operand is far cheaper than running the general kernel.
     k_strided = (lay == N.ROW_MAJOR) if sparse_first else (lay == N.COL_MAJOR)
-    if k_strided and store_layout == N.COMPRESSED_PANEL and dense.numel() // k <= 16:
-        # a few dense columns: the one-pass kernel for them wants k contiguous, and the operand is tiny
+    if k_strided and store_layout == N.COMPRESSED_PANEL and dense.numel() // k <= 64:
+        # a few dense columns: the kernels for them want k contiguous, and the operand is tiny
         flipped = (dense if sparse_first else dense.t()).t().contiguous()       # [j, k]
         dense = flipped.t() if sparse_first else flipped
         lay, ld = N.layout_of(dense)
