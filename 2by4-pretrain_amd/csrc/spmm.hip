@@ -789,8 +789,9 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
 // LDS at the end (added in wave order).  In the panel layout the A fragments of
 // 16 adjacent rows are 1 KB of contiguous memory (16 bytes per lane) and their index words 128
 // (256) contiguous bytes; the dense fragment is 64 contiguous bytes from each of the 16 dense rows,
-// twice.  Loads are issued 16 panels at a time (about 16 KB of the sparse operand per wave in
-// flight): left to itself the compiler waits for each panel's loads before it issues the next.
+// twice.  Loads are issued 8 panels at a time into one of two register sets, the next batch while
+// the current one is multiplied (up to 16 KB of the sparse operand per wave in flight): left to
+// itself the compiler waits for each panel's loads before it issues the next.
 // ------------------------------------------------------------------------------------------
 constexpr int kNarrowMaxDense = 16;
 constexpr int kNarrowWaves = 4;
@@ -802,7 +803,7 @@ spmm_narrow(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_
             OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
   constexpr int KSTEP = mma16<T>::KSTEP;     // dense k per panel = per instruction
   constexpr int M_ROW = KSTEP / 8;           // metadata bytes per row per panel
-  constexpr int BATCH = 16;
+  constexpr int BATCH = 8;                   // panels per load batch; two batches are in flight
   using acc_t = typename mma16<T>::acc_t;
   __shared__ acc_t s_acc[kNarrowWaves - 1][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, lk = lane >> 4;
@@ -818,26 +819,40 @@ spmm_narrow(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_
   acc_t acc[2];                              // two chains, so that consecutive instructions do not wait on each other
 #pragma unroll
   for (int r = 0; r < 4; r++) { acc[0][r] = 0; acc[1][r] = 0; }
-  for (int64_t p = p_begin; p < p_end; p += BATCH) {
-    int4v af[BATCH], lo[BATCH], hi[BATCH];
-    int idx[BATCH];
+  // two register sets: the loads of the next batch are in flight while the current one is multiplied
+  int4v af[2][BATCH], lo[2][BATCH], hi[2][BATCH];
+  int idx[2][BATCH];
+  auto load_batch = [&](int set, int64_t p) {
 #pragma unroll
     for (int u = 0; u < BATCH; u++) {
       const int64_t pp = p + u < p_end ? p + u : p_end - 1;     // past the end: re-read the last panel, multiply by zero
-      af[u] = __builtin_nontemporal_load(reinterpret_cast<const int4v*>(av + pp * a_step));
-      if constexpr (sizeof(T) == 2) idx[u] = *reinterpret_cast<const uint16_t*>(am + pp * m_step);
-      else idx[u] = *reinterpret_cast<const int*>(am + pp * m_step);
-      lo[u] = *reinterpret_cast<const int4v*>(bp + pp * 128);
-      hi[u] = *reinterpret_cast<const int4v*>(bp + pp * 128 + 64);
+      af[set][u] = __builtin_nontemporal_load(reinterpret_cast<const int4v*>(av + pp * a_step));
+      if constexpr (sizeof(T) == 2) idx[set][u] = *reinterpret_cast<const uint16_t*>(am + pp * m_step);
+      else idx[set][u] = *reinterpret_cast<const int*>(am + pp * m_step);
+      lo[set][u] = *reinterpret_cast<const int4v*>(bp + pp * 128);
+      hi[set][u] = *reinterpret_cast<const int4v*>(bp + pp * 128 + 64);
     }
-    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto multiply_batch = [&](int set, int64_t p) {
 #pragma unroll
     for (int u = 0; u < BATCH; u++) {
-      if (p + u >= p_end) af[u] = int4v{0, 0, 0, 0};
-      const int8v bfrag = {lo[u][0], lo[u][1], lo[u][2], lo[u][3], hi[u][0], hi[u][1], hi[u][2], hi[u][3]};
-      acc[u & 1] = mma16<T>::template run<0>(af[u], bfrag, acc[u & 1], idx[u]);
+      const int4v a = p + u < p_end ? af[set][u] : int4v{0, 0, 0, 0};
+      const int8v bfrag = {lo[set][u][0], lo[set][u][1], lo[set][u][2], lo[set][u][3], hi[set][u][0], hi[set][u][1], hi[set][u][2], hi[set][u][3]};
+      acc[u & 1] = mma16<T>::template run<0>(a, bfrag, acc[u & 1], idx[set][u]);
     }
+  };
+  if (p_begin < p_end) load_batch(0, p_begin);
+  for (int64_t p = p_begin; p < p_end; p += 2 * BATCH) {
+    if (p + BATCH < p_end) load_batch(1, p + BATCH);
+    __builtin_amdgcn_sched_barrier(0);       // keep the loads ahead of the instructions that wait for the previous batch
+    multiply_batch(0, p);
     __builtin_amdgcn_sched_barrier(0);
+    if (p + BATCH < p_end) {
+      if (p + 2 * BATCH < p_end) load_batch(0, p + 2 * BATCH);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply_batch(1, p + BATCH);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   acc_t sum = acc[0] + acc[1];
   if (wave > 0) s_acc[wave - 1][lane] = sum;
