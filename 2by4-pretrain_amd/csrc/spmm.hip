@@ -15,6 +15,7 @@
 //      range shifted by K/2
 //   D: 16x16: column l%16, rows 4*(l/16)+r;  32x32: column l%32, rows 8*(r/4) + 4*(l/32) + r%4
 #include "tf24_common.hpp"
+#include <algorithm>
 #include <type_traits>
 
 namespace tf24 {
@@ -275,7 +276,7 @@ struct TileCfgT {
   static constexpr int TI = 4, TJ = TJ_;         // 32x32 instructions per wave
   static constexpr int WI = 32 * TI, WJ = 32 * TJ;
   static constexpr int BI = WI * WAVES_I, BJ = WJ * WAVES_J;
-  static_assert(BI == 256 && (BJ == 256 || BJ == 64), "stage buffers are sized for 256 x 256 and 256 x 64 tiles");
+  static_assert(BI == 256 && (BJ == 256 || BJ == 128 || BJ == 64), "stage buffers are sized for 256-row tiles of 256, 128 or 64 columns");
   static constexpr int KB = 128;                 // bytes of dense k per row per stage
   static constexpr int STEPS = KB / 64;          // instruction steps per stage
   static constexpr int A_ROW = KB / 2;           // LDS bytes per row per stage: compressed values
@@ -288,6 +289,8 @@ using TiledCfg = TileCfgT<4, 2>;
 // 256 x 64 tiles, two waves: for dense operands of at most 64 columns (a few dozen tokens), where a
 // 256-wide tile would copy and multiply clamped columns.  26 KB per stage, two blocks per CU.
 using SlimCfg = TileCfgT<1, 2>;
+// 256 x 128 tiles, four waves: dense operands of 65 to 128 columns
+using MidCfg = TileCfgT<2, 2>;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -710,10 +713,18 @@ spmm_reduce_splits(const float* __restrict__ partial, int splits, int tiles_i, i
   for (int slab = blockIdx.y; slab < NSLAB; slab += gridDim.y) {
     const int ti = slab / (C::TJ * 4), tj = (slab / 4) % C::TJ, g = slab % 4;
     if (j0 + wj * C::WJ + tj * 32 >= n_dense) continue;          // the whole 32-column slab lies past the dense operand
+    // the pieces are loaded eight at a time (independent loads in flight) and added in piece order
     Acc4 sum = {0, 0, 0, 0};
-    for (int sp = 0; sp < splits; sp++) {
-      const float* base = partial + ((int64_t)sp * ntiles + tile) * (C::BI * C::BJ);
-      sum += *reinterpret_cast<const Acc4*>(base + ((int64_t)slab * C::THREADS + tid) * 4);
+    const float* first = partial + (int64_t)tile * (C::BI * C::BJ) + ((int64_t)slab * C::THREADS + tid) * 4;
+    const int64_t piece = (int64_t)ntiles * (C::BI * C::BJ);
+    for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+      Acc4 part[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        part[u] = *reinterpret_cast<const Acc4*>(first + (int64_t)min(sp0 + u, splits - 1) * piece);
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        if (sp0 + u < splits) sum += part[u];
     }
     const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
     const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
@@ -737,7 +748,7 @@ int choose_splits(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspac
   const int64_t tiles = ((n_sparse + C::BI - 1) / C::BI) * ((n_dense + C::BJ - 1) / C::BJ);
   const int64_t nstages = k * (int64_t)sizeof(T) / C::KB;
   if (tiles >= 160) return 1;
-  int64_t splits = 256 / tiles;
+  int64_t splits = 192 / tiles;              // measured: filling all 256 CUs costs more in partial tiles than it gains
   if (splits > nstages / 4) splits = nstages / 4;
   if (splits > 16) splits = 16;
   while (splits > 1 && splits * tiles * C::BI * C::BJ * 4 > workspace_bytes) splits--;
@@ -770,7 +781,7 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
     else launch(std::false_type{}, std::false_type{});
   }
   if (splits > 1) {
-    dim3 rgrid((unsigned)(tiles_i * tiles_j), 8);
+    dim3 rgrid((unsigned)(tiles_i * tiles_j), C::TI * C::TJ * 4);      // one accumulator group of the tile per block
     if (jm)
       hipLaunchKernelGGL((spmm_reduce_splits<typename mma32<T>::acc4_t, OutT, true, C>), rgrid, dim3(C::THREADS), 0, s, (const float*)workspace, splits, tiles_i, tiles_j,
                          n_sparse, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act);
@@ -912,13 +923,17 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
   // the tiled kernel reads a k-strided dense operand through transposing LDS reads (16-bit types only)
   // (also for a narrow dense operand: with its k pieces the tiled kernel beats the general one from 8 columns on)
   const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64;
-  // at most 16 dense columns: one pass over the compressed operand, no staging
-  const bool narrow = panel && b_layout == TF24_ROW_MAJOR && n_dense <= kNarrowMaxDense;
-  // up to 64 dense columns: the tiled kernel on 256 x 64 tiles
+  // up to 64 dense columns: the tiled kernel on 256 x 64 tiles; up to 128: on 256 x 128 tiles
   const bool slim = tiled && b_layout == TF24_ROW_MAJOR && n_dense <= SlimCfg::BJ;
+  const bool mid = tiled && b_layout == TF24_ROW_MAJOR && n_dense <= MidCfg::BJ;
+  // at most 8 dense columns: one pass over the compressed operand, no staging; up to 16 when the
+  // tiled kernel cannot cut k into pieces (no workspace), which it needs to fill the chip
+  const bool narrow = panel && b_layout == TF24_ROW_MAJOR &&
+                      (n_dense <= 8 || (n_dense <= kNarrowMaxDense && !(slim && workspace)));
   if constexpr (std::is_same<T, i8_t>::value) {        // integer product: int32 accumulators, results and bias
     if (narrow) return launch_narrow<T, int32_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
     if (slim) return launch_tiled<T, int32_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+    if (mid) return launch_tiled<T, int32_t, MidCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     if (tiled) return launch_tiled<T, int32_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     return launch_general<T, int32_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   } else {
@@ -934,6 +949,13 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
       case TF24_F16: return launch_tiled<T, f16_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
       case TF24_BF16: return launch_tiled<T, bf16_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
       case TF24_F32: return launch_tiled<T, float, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+    }
+  }
+  if (mid) {
+    switch (out_dtype) {
+      case TF24_F16: return launch_tiled<T, f16_t, MidCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_BF16: return launch_tiled<T, bf16_t, MidCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
+      case TF24_F32: return launch_tiled<T, float, MidCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     }
   }
   if (tiled) {
@@ -982,22 +1004,25 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
   return TF24_OK;
 }
 
+namespace tf24 {
+namespace {
+template <typename C>
+int64_t split_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense) {
+  const int64_t big = (int64_t)1 << 40;
+  const int splits = is_8bit(dtype) ? choose_splits<e4m3_t, C>(n_sparse, k, n_dense, big) : choose_splits<f16_t, C>(n_sparse, k, n_dense, big);
+  if (splits < 2) return 0;
+  const int64_t tiles = ((n_sparse + C::BI - 1) / C::BI) * ((n_dense + C::BJ - 1) / C::BJ);
+  return splits * tiles * C::BI * C::BJ * 4;
+}
+}  // namespace
+}  // namespace tf24
+
+// the float32 partial tiles of the k pieces, for whichever tile configuration the shape selects
 extern "C" int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense) {
   using namespace tf24;
-  const int64_t big = (int64_t)1 << 40;
-  int splits;
-  if (is_8bit(dtype)) splits = choose_splits<e4m3_t, TiledCfg>(n_sparse, k, n_dense, big);
-  else splits = choose_splits<f16_t, TiledCfg>(n_sparse, k, n_dense, big);
-  int64_t bytes = 0;
-  if (splits >= 2) {
-    const int64_t tiles = ((n_sparse + TiledCfg::BI - 1) / TiledCfg::BI) * ((n_dense + TiledCfg::BJ - 1) / TiledCfg::BJ);
-    bytes = splits * tiles * TiledCfg::BI * TiledCfg::BJ * 4;
-  }
-  if (n_dense <= SlimCfg::BJ) {              // the 64-wide tile's k pieces
-    const int ss = is_8bit(dtype) ? choose_splits<e4m3_t, SlimCfg>(n_sparse, k, n_dense, big) : choose_splits<f16_t, SlimCfg>(n_sparse, k, n_dense, big);
-    const int64_t need = ss >= 2 ? (int64_t)ss * ((n_sparse + SlimCfg::BI - 1) / SlimCfg::BI) * SlimCfg::BI * SlimCfg::BJ * 4 : 0;
-    if (need > bytes) bytes = need;
-  }
+  int64_t bytes = split_bytes<TiledCfg>(dtype, n_sparse, k, n_dense);
+  if (n_dense <= MidCfg::BJ) bytes = std::max(bytes, split_bytes<MidCfg>(dtype, n_sparse, k, n_dense));
+  if (n_dense <= SlimCfg::BJ) bytes = std::max(bytes, split_bytes<SlimCfg>(dtype, n_sparse, k, n_dense));
   return bytes;
 }
 

@@ -800,11 +800,13 @@ def test_int8_spmm_extreme_values(cuda):
     assert out.cpu().equal(torch.full((m, n), 16384 * (k // 2), dtype=torch.int32))
 
 
-@pytest.mark.parametrize("dtype,m", [(F16, 8), (F16, 24), (BF16, 40), (E4M3, 16), (torch.int8, 16)])
+@pytest.mark.parametrize("dtype,m", [(F16, 8), (BF16, 8), (F16, 24), (BF16, 40), (E4M3, 16), (torch.int8, 16),
+                                     (F16, 72), (BF16, 128), (E4M3, 80), (torch.int8, 128)])
 @pytest.mark.parametrize("k", [512, 4096])
 def test_spmm_narrow_dense_operand(cuda, dtype, m, k):
-    """A handful of dense columns against a tall sparse operand: the tiled kernel (with k pieces at
-    k = 4096) whose partial tiles only cover the live 32-column slabs; every operand position and layout."""
+    """A handful of dense columns against a tall sparse operand: 8 columns take the one-pass kernel,
+    up to 64 and up to 128 the tiled kernel on 256 x 64 and 256 x 128 tiles (with k pieces, whose
+    partial tiles only cover the live 32-column slabs); every operand position and layout."""
     import sparse
     n = 320
     if dtype == torch.int8:
@@ -824,11 +826,38 @@ def test_spmm_narrow_dense_operand(cuda, dtype, m, k):
     assert same(torch.mm(s, xg.t().contiguous()), ref.t())
 
 
+@pytest.mark.parametrize("dtype", [F16, E4M3, torch.int8])
+@pytest.mark.parametrize("n,k", [(320, 1024), (8192, 1408 * 2)])
+def test_spmm_16_columns_without_workspace(cuda, dtype, n, k):
+    """Through the C ABI with no workspace the tiled kernel cannot cut k into pieces, and 16 dense
+    columns take the one-pass kernel (four waves per block at 320 rows, one at 8192)."""
+    import sparse
+    from sparse import _native as N
+    m = 16
+    if dtype == torch.int8:
+        w, x = _int8((n, k), 141, -3, 4), _int8((m, k), 142, -3, 4)
+        ref = oracle.spmm_ref_int(x, torch.where(oracle.prune24_mask(w.float()), w, torch.zeros_like(w)))
+        s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+        out_dtype, out_code = torch.int32, N.I32
+    else:
+        w, x = _small_ints((n, k), 141, -2, 3).to(dtype), _small_ints((m, k), 142, -2, 3).to(dtype)
+        ref = oracle.spmm_ref(x.float(), torch.where(oracle.prune24_mask(w.float()), w.float(), torch.zeros(())))
+        s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+        out_dtype, out_code = torch.float32, N.F32
+    xg = x.to(cuda)
+    out = torch.empty(m, n, dtype=out_dtype, device=cuda)
+    N.check(N.lib().tf24_spmm(s._store_values.data_ptr(), s._store_meta.data_ptr(), N.COMPRESSED_PANEL, N.operand_code(dtype), n, k,
+                              xg.data_ptr(), N.ROW_MAJOR, k, m, out.data_ptr(), out_code, N.COL_MAJOR, n, None, 1.0, 0,
+                              None, 0, N.stream_ptr()))
+    torch.cuda.synchronize()
+    assert out.cpu().to(torch.float64).equal(ref.to(torch.float64))
+
+
 @pytest.mark.parametrize("dtype", [F16, E4M3])
 def test_spmm_narrow_one_wave_per_block(cuda, dtype):
-    """Many sparse rows and at most 16 dense columns: the narrow kernel runs one wave per 16-row block
-    (fewer rows split k over four waves: test_spmm_narrow_dense_operand); k not a multiple of its
-    16-panel load batch."""
+    """Many sparse rows and few dense columns (16 through the tiled kernel's 64-wide tiles, 8 through the
+    one-pass kernel with one wave per 16-row block; fewer rows split k over four waves:
+    test_spmm_narrow_dense_operand); k not a multiple of the one-pass kernel's load batches."""
     import sparse
     n, k, m = 8192, 1408 if dtype == F16 else 2816, 16
     w, x = _small_ints((n, k), 131, -2, 3).to(dtype), _small_ints((m, k), 132, -2, 3).to(dtype)
