@@ -14,8 +14,8 @@ import torch
 import torch.nn.functional as F
 from torch import autograd, nn
 
-from .semi_structured import (SparseSemiStructuredTensor, _spmm, to_sparse_semi_structured, to_sparse_semi_structured_pair,
-                              to_sparse_semi_structured_with_row_sums)
+from .semi_structured import (SparseSemiStructuredTensor, _dense_times_sparse_t, _spmm, to_sparse_semi_structured,
+                              to_sparse_semi_structured_pair, to_sparse_semi_structured_with_row_sums)
 from .transposable_semi_structured import TransposableSparse
 
 __all__ = ["SparseLinearTranspose", "sparse_linear_transpose"]
@@ -40,10 +40,9 @@ class sparse_linear_transpose(autograd.Function):
             ctx.shape = input.shape
             ctx.weight_dtype = weight.dtype
             input = input.view(-1, input.shape[-1])
-            if bias is None:
-                output = torch.mm(input, weight_sparse.t())
-            else:
-                output = torch.addmm(bias, input, weight_sparse.t())      # bias added in the matmul epilogue
+            # = torch.mm(input, weight_sparse.t()) / torch.addmm(bias, input, weight_sparse.t()) (README.md:176-179)
+            # called directly; the bias is added in the matmul epilogue
+            output = _dense_times_sparse_t(input, weight_sparse, bias)
             return output.view(*ctx.shape[:-1], -1)
 
     @staticmethod
@@ -57,7 +56,7 @@ class sparse_linear_transpose(autograd.Function):
             if grad_output.dtype != input.dtype:
                 grad_output = grad_output.to(input.dtype)
             if ctx.needs_input_grad[0]:
-                grad_input = torch.mm(grad_output, weight_T.t()).view(ctx.shape)
+                grad_input = _dense_times_sparse_t(grad_output, weight_T).view(ctx.shape)      # = torch.mm(grad_output, weight_T.t())
             if ctx.needs_input_grad[1]:
                 input = input.view(-1, input.shape[-1])
                 if ctx.needs_input_grad[4]:
