@@ -1,23 +1,33 @@
 // Compressed 2:4 -> dense for gfx950.  Lane owns 8 dense outputs (two groups): loads its 4 kept
 // values and one metadata byte, stores 8 elements with one vector store.
 #include "tf24_common.hpp"
+#include <type_traits>
 
 namespace tf24 {
 namespace {
 
 constexpr int kThreads = 256;
 
-template <typename T>
+// canonical: units in row-major order.  panel: a block covers 8 rows x 32 units (a wave 2 rows),
+// blocks numbered along k first, so that a wave reads the two rows' adjacent 64-byte pieces of 4
+// (2) panels as whole cache lines and writes 512 contiguous bytes per row.
+template <typename T, bool PANEL>
 __global__ void __launch_bounds__(kThreads)
 decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta, int64_t total_units, int64_t m, int64_t k,
-                  bool panel, T* __restrict__ dense) {
-  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;   // unit = 8 dense elements, row-major order
-  if (u >= total_units) return;
-  int64_t src = u;
-  if (panel) {        // [k/KP][m][KP/8 units]
+                  uint32_t chunks, T* __restrict__ dense) {
+  int64_t u, src;
+  if constexpr (PANEL) {        // [k/KP][m][KP/8 units]
     constexpr int UPP = (128 / (int)sizeof(T)) / 8;
-    const int64_t upr = k >> 3, row = u / upr, col8 = u - row * upr;
+    const int64_t upr = k >> 3;
+    const uint32_t by = blockIdx.x / chunks, bx = blockIdx.x - by * chunks;        // chunks = 32-unit pieces of a row
+    const int64_t col8 = (int64_t)bx * 32 + (threadIdx.x & 31), row = (int64_t)by * 8 + (threadIdx.x >> 5);
+    if (col8 >= upr || row >= m) return;
+    u = row * upr + col8;
     src = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
+  } else {
+    u = (int64_t)blockIdx.x * kThreads + threadIdx.x;   // unit = 8 dense elements, row-major order
+    if (u >= total_units) return;
+    src = u;
   }
   Pack<T, 4> v;
   v.load_stream(values + src * 4);
@@ -41,27 +51,47 @@ decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta
 template <typename T>
 int launch(const void* values, const void* meta, bool panel, int64_t m, int64_t k, void* dense, hipStream_t s) {
   const int64_t total = m * (k / 8);
-  dim3 grid((unsigned)((total + kThreads - 1) / kThreads));
-  hipLaunchKernelGGL((decompress_kernel<T>), grid, dim3(kThreads), 0, s, (const T*)values, (const uint8_t*)meta, total, m, k, panel, (T*)dense);
+  if (panel) {
+    const int64_t chunks = (k / 8 + 31) / 32, blocks = chunks * ((m + 7) / 8);
+    if (blocks > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "tf24_decompress: matrix too large");
+    hipLaunchKernelGGL((decompress_kernel<T, true>), dim3((unsigned)blocks), dim3(kThreads), 0, s, (const T*)values, (const uint8_t*)meta, total, m, k,
+                       (uint32_t)chunks, (T*)dense);
+  } else {
+    dim3 grid((unsigned)((total + kThreads - 1) / kThreads));
+    hipLaunchKernelGGL((decompress_kernel<T, false>), grid, dim3(kThreads), 0, s, (const T*)values, (const uint8_t*)meta, total, m, k, 0u, (T*)dense);
+  }
   return check_launch("tf24_decompress");
 }
 
 // Canonical <-> panel storage of a compressed operand.  Per row and panel the 64 value bytes and the
-// KP/8 metadata bytes are the same in both forms, only their place differs: a lane moves 16 value
-// bytes, the first lanes of a row-panel also its metadata.
+// KP/8 metadata bytes are the same in both forms, only their place differs.  A block moves 8 rows x
+// 8 panels: a wave the values of 2 rows x 8 panels, 16 bytes per lane (canonical side: 512
+// contiguous bytes per row; panel side: the two rows' adjacent pieces, one cache line per panel);
+// the first wave also the 64 metadata pieces, lane = (row, panel) (64- or 128-byte runs on both sides).
+template <int META_BYTES>
 __global__ void __launch_bounds__(kThreads)
-repack_kernel(const uint8_t* __restrict__ vin, const uint8_t* __restrict__ min_, int64_t m, int64_t panels, int meta_bytes,
+repack_kernel(const uint8_t* __restrict__ vin, const uint8_t* __restrict__ min_, int64_t m, int64_t panels, uint32_t chunks,
               bool to_panel, uint8_t* __restrict__ vout, uint8_t* __restrict__ mout) {
-  const int64_t t = (int64_t)blockIdx.x * kThreads + threadIdx.x;   // 4 lanes per (row, panel), canonical order
-  const int64_t chunk = t >> 2;
-  const int part = (int)(t & 3);
-  if (chunk >= m * panels) return;
-  const int64_t row = chunk / panels, p = chunk - row * panels;
-  const int64_t canon = row * panels + p, panel = p * m + row;
-  const int64_t src = to_panel ? canon : panel, dst = to_panel ? panel : canon;
-  *reinterpret_cast<uint4*>(vout + dst * 64 + part * 16) = *reinterpret_cast<const uint4*>(vin + src * 64 + part * 16);
-  if (part * 8 < meta_bytes)
-    *reinterpret_cast<uint2*>(mout + dst * meta_bytes + part * 8) = *reinterpret_cast<const uint2*>(min_ + src * meta_bytes + part * 8);
+  const uint32_t by = blockIdx.x / chunks, bx = blockIdx.x - by * chunks;          // chunks = 8-panel pieces of a row
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  {
+    const int part = lane & 3;
+    const int64_t p = (int64_t)bx * 8 + ((lane >> 2) & 7), row = (int64_t)by * 8 + wave * 2 + (lane >> 5);
+    if (p < panels && row < m) {
+      const int64_t canon = row * panels + p, panel = p * m + row;
+      const int64_t src = to_panel ? canon : panel, dst = to_panel ? panel : canon;
+      *reinterpret_cast<uint4*>(vout + dst * 64 + part * 16) = *reinterpret_cast<const uint4*>(vin + src * 64 + part * 16);
+    }
+  }
+  if (wave == 0) {
+    const int64_t p = (int64_t)bx * 8 + (lane & 7), row = (int64_t)by * 8 + (lane >> 3);
+    if (p < panels && row < m) {
+      const int64_t canon = row * panels + p, panel = p * m + row;
+      const int64_t src = to_panel ? canon : panel, dst = to_panel ? panel : canon;
+      using Piece = typename std::conditional<META_BYTES == 16, uint4, uint2>::type;
+      *reinterpret_cast<Piece*>(mout + dst * META_BYTES) = *reinterpret_cast<const Piece*>(min_ + src * META_BYTES);
+    }
+  }
 }
 
 }  // namespace
@@ -77,12 +107,17 @@ extern "C" int tf24_repack(const void* values_in, const void* meta_in, int dtype
   if (from_layout != TF24_COMPRESSED_CANONICAL && from_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, from_layout);
   if (!values_in || !meta_in || !values_out || !meta_out) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
   if (values_in == values_out || meta_in == meta_out) return fail(TF24_ERR_ARG, "%s: in-place conversion is not supported", fn);
-  if (((uintptr_t)values_in | (uintptr_t)values_out) % 16 || ((uintptr_t)meta_in | (uintptr_t)meta_out) % 8)
-    return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte and metadata 8-byte aligned", fn);
-  const int64_t panels = k / kp, threads = m * panels * 4;
-  dim3 grid((unsigned)((threads + kThreads - 1) / kThreads));
-  hipLaunchKernelGGL(repack_kernel, grid, dim3(kThreads), 0, (hipStream_t)stream, (const uint8_t*)values_in, (const uint8_t*)meta_in, m, panels,
-                     (int)(kp / 8), from_layout == TF24_COMPRESSED_CANONICAL, (uint8_t*)values_out, (uint8_t*)meta_out);
+  if (((uintptr_t)values_in | (uintptr_t)values_out) % 16 || ((uintptr_t)meta_in | (uintptr_t)meta_out) % (kp / 8))
+    return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte and metadata %lld-byte aligned", fn, (long long)(kp / 8));
+  const int64_t panels = k / kp, chunks = (panels + 7) / 8, blocks = chunks * ((m + 7) / 8);
+  if (blocks > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "%s: matrix too large", fn);
+  const bool to_panel = from_layout == TF24_COMPRESSED_CANONICAL;
+  if (kp == 128)
+    hipLaunchKernelGGL(repack_kernel<16>, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint8_t*)values_in, (const uint8_t*)meta_in,
+                       m, panels, (uint32_t)chunks, to_panel, (uint8_t*)values_out, (uint8_t*)meta_out);
+  else
+    hipLaunchKernelGGL(repack_kernel<8>, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint8_t*)values_in, (const uint8_t*)meta_in,
+                       m, panels, (uint32_t)chunks, to_panel, (uint8_t*)values_out, (uint8_t*)meta_out);
   return check_launch(fn);
 }
 
