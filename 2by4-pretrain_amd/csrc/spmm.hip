@@ -755,6 +755,24 @@ int choose_splits(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspac
   return splits < 2 ? 1 : (int)splits;
 }
 
+// Time estimate of the tiled kernel on one tile configuration, to choose between 256 x 256 and
+// 256 x 128 tiles for operands of a few hundred dense columns: rounds of at most 256 blocks (one per
+// CU) x stages per block x the stage time measured for that configuration (0.95 us for 256 x 256
+// tiles, 0.55 us for 256 x 128), plus, with k pieces, the partial tiles written and read at
+// 4.5 TB/s and the second launch.  On W[11008, 4096], W[4096, 11008] and W[8192, 8192] with 256 to
+// 1536 dense columns it picks the faster configuration in every case measured (up to 30 % apart).
+struct TileCost { int64_t blocks; double us; };
+template <typename T, typename C>
+TileCost tile_cost(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspace_bytes, double stage_us) {
+  const int64_t tiles = ((n_sparse + C::BI - 1) / C::BI) * ((n_dense + C::BJ - 1) / C::BJ);
+  const int64_t nstages = k * (int64_t)sizeof(T) / C::KB;
+  const int64_t splits = workspace_bytes > 0 ? choose_splits<T, C>(n_sparse, k, n_dense, workspace_bytes) : 1;
+  const int64_t blocks = tiles * splits, rounds = (blocks + 255) / 256;
+  double us = (double)rounds * (double)((nstages + splits - 1) / splits) * stage_us;
+  if (splits > 1) us += 2.0 * (double)(splits * tiles * C::BI * C::BJ * 4) / 4.5e6 + 3.0;
+  return {blocks, us};
+}
+
 template <typename T, typename OutT, typename C>
 int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
@@ -925,7 +943,12 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
   const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64;
   // up to 64 dense columns: the tiled kernel on 256 x 64 tiles; up to 128: on 256 x 128 tiles
   const bool slim = tiled && b_layout == TF24_ROW_MAJOR && n_dense <= SlimCfg::BJ;
-  const bool mid = tiled && b_layout == TF24_ROW_MAJOR && n_dense <= MidCfg::BJ;
+  // wider operands that still fit one round of 256 x 128 tiles take those when the estimate below says so
+  const int64_t ws_bytes = workspace ? workspace_bytes : 0;
+  const bool mid = tiled && b_layout == TF24_ROW_MAJOR &&
+                   (n_dense <= MidCfg::BJ ||
+                    (tile_cost<T, MidCfg>(n_sparse, k, n_dense, ws_bytes, 0.55).blocks <= 256 &&
+                     tile_cost<T, MidCfg>(n_sparse, k, n_dense, ws_bytes, 0.55).us < tile_cost<T, TiledCfg>(n_sparse, k, n_dense, ws_bytes, 0.95).us));
   // at most 8 dense columns: one pass over the compressed operand, no staging; up to 16 when the
   // tiled kernel cannot cut k into pieces (no workspace), which it needs to fill the chip
   const bool narrow = panel && b_layout == TF24_ROW_MAJOR &&
@@ -1021,7 +1044,7 @@ int64_t split_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense) {
 extern "C" int64_t tf24_spmm_workspace_bytes(int dtype, int64_t n_sparse, int64_t k, int64_t n_dense) {
   using namespace tf24;
   int64_t bytes = split_bytes<TiledCfg>(dtype, n_sparse, k, n_dense);
-  if (n_dense <= MidCfg::BJ) bytes = std::max(bytes, split_bytes<MidCfg>(dtype, n_sparse, k, n_dense));
+  bytes = std::max(bytes, split_bytes<MidCfg>(dtype, n_sparse, k, n_dense));
   if (n_dense <= SlimCfg::BJ) bytes = std::max(bytes, split_bytes<SlimCfg>(dtype, n_sparse, k, n_dense));
   return bytes;
 }
