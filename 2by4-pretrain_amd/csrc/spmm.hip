@@ -811,19 +811,21 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
 }
 
 // ------------------------------------------------------------------------------------------
-// Narrow kernel: at most 16 dense columns (decoding a few tokens against a large sparse weight).
-// The product is bound by one pass over the compressed operand, so nothing is staged: a block owns
-// 16 sparse rows; its waves (one when the rows alone give enough blocks to fill the chip, otherwise
-// up to four, each taking a share of the k range) run one V_SMFMAC_*_16X16 per panel and meet in
-// LDS at the end (added in wave order).  In the panel layout the A fragments of
-// 16 adjacent rows are 1 KB of contiguous memory (16 bytes per lane) and their index words 128
-// (256) contiguous bytes; the dense fragment is 64 contiguous bytes from each of the 16 dense rows,
-// twice.  Loads are issued 8 panels at a time into one of two register sets, the next batch while
-// the current one is multiplied (up to 16 KB of the sparse operand per wave in flight): left to
-// itself the compiler waits for each panel's loads before it issues the next.
+// Narrow kernels: at most 16 dense columns (decoding a few tokens against a large sparse weight).
+// The product is bound by one pass over the compressed operand, so the sparse operand is not
+// staged: a wave streams the A fragments of 16 sparse rows straight into registers (in the panel
+// layout 1 KB of contiguous memory per panel, 16 bytes per lane, and their index words 128 (256)
+// contiguous bytes) and runs one V_SMFMAC_*_16X16 per panel.  Loads are issued a batch of panels at
+// a time into one of two register sets, the next batch while the current one is multiplied: left
+// to itself the compiler waits for each panel's loads before it issues the next.
+// Fewer than 512 row blocks (spmm_narrow): a block owns 16 rows, its up to four waves each take a
+// share of the k range, read their dense fragments from global memory (64 contiguous bytes from
+// each of the 16 dense rows, twice) and meet in LDS at the end (added in wave order).
+// From 512 row blocks on (spmm_narrow_shared): see there.
 // ------------------------------------------------------------------------------------------
 constexpr int kNarrowMaxDense = 16;
 constexpr int kNarrowWaves = 4;
+constexpr int kNarrowSharedMin = 160;      // workgroups of four 16-row blocks below which two blocks per workgroup are faster
 
 template <typename T, typename OutT, bool C_JMAJOR>
 __global__ void __launch_bounds__(64 * kNarrowWaves)
@@ -901,13 +903,146 @@ spmm_narrow(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_
   }
 }
 
+// Narrow kernel for many sparse rows: the NW (2 or 4) waves of a block own adjacent 16-row blocks and
+// share the dense operand through LDS, 16 panels (a chunk) at a time in two buffers, so that the
+// only loads of the main loop are the sparse operand's: the one-wave form above sends every wave's
+// dense fragments through L1 (twice the requests of its share of the sparse operand), and the
+// kernel is bound by the number of requests in flight, not by bytes.  LDS holds
+// [panel][column][128 bytes] with the 16-byte pieces of a column XOR-swizzled by column / 2, so the
+// 16 lanes that read one piece position of 16 columns hit 16 different bank groups.
+// NC = dense columns kept in LDS (8 or 16).
+template <typename T, typename OutT, bool C_JMAJOR, int NC, int NW>
+__global__ void __launch_bounds__(64 * NW)
+spmm_narrow_shared(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
+                   const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
+                   OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act) {
+  constexpr int KSTEP = mma16<T>::KSTEP;
+  constexpr int M_ROW = KSTEP / 8;
+  constexpr int CH = 16;                              // panels per chunk
+  constexpr int THREADS = 64 * NW;
+  constexpr int PIECES = NC * CH * 8 / THREADS;       // 16-byte pieces of the dense chunk per thread (4 to 16)
+  using acc_t = typename mma16<T>::acc_t;
+  __shared__ __attribute__((aligned(16))) uint8_t s_b[2][CH * NC * 128];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lk = lane >> 4;
+  const int64_t blocks16 = n_sparse / 16;
+  const int64_t rb = (int64_t)blockIdx.x * NW + wave;
+  const bool active = rb < blocks16;
+  const int64_t i0 = (active ? rb : blocks16 - 1) * 16;
+  const int64_t npanels = k / KSTEP;
+  const int nchunks = (int)((npanels + CH - 1) / CH);
+  const uint8_t* av = a_values + (i0 + li) * 64 + lk * 16;
+  const uint8_t* am = a_meta + (i0 + li) * M_ROW + lk * (M_ROW / 4);
+  const int64_t a_step = n_sparse * 64, m_step = n_sparse * M_ROW;
+  // dense chunk: thread's piece q = tid + THREADS j -> column q / (CH * 8), piece q % (CH * 8) of the column's 2 KB
+  const uint8_t* bsrc[PIECES];
+  int bdst[PIECES], bwithin[PIECES];
+#pragma unroll
+  for (int j = 0; j < PIECES; j++) {
+    const int q = tid + THREADS * j, col = q / (CH * 8), within = q % (CH * 8);
+    const int64_t gcol = col < n_dense ? col : n_dense - 1;
+    bsrc[j] = b + gcol * ldb_bytes + within * 16;
+    bwithin[j] = within;
+    bdst[j] = ((within >> 3) * NC + col) * 128 + (((within & 7) ^ ((col >> 1) & 7)) * 16);
+  }
+  const int64_t row_bytes = npanels * 128;             // bytes of one dense row
+  const int colr = li < n_dense ? li : (int)n_dense - 1;
+  const int rd_lo = colr * 128 + ((lk ^ ((colr >> 1) & 7)) * 16), rd_hi = colr * 128 + (((lk + 4) ^ ((colr >> 1) & 7)) * 16);
+  acc_t acc[2];
+#pragma unroll
+  for (int r = 0; r < 4; r++) { acc[0][r] = 0; acc[1][r] = 0; }
+  int4v af[2][CH], breg[PIECES];
+  int idx[2][CH];
+  auto load_a = [&](int set, int chunk) {
+#pragma unroll
+    for (int u = 0; u < CH; u++) {
+      const int64_t p = (int64_t)chunk * CH + u;
+      const int64_t pp = p < npanels ? p : npanels - 1;          // past the end: re-read the last panel, multiply by zero
+      af[set][u] = __builtin_nontemporal_load(reinterpret_cast<const int4v*>(av + pp * a_step));
+      if constexpr (sizeof(T) == 2) idx[set][u] = *reinterpret_cast<const uint16_t*>(am + pp * m_step);
+      else idx[set][u] = *reinterpret_cast<const int*>(am + pp * m_step);
+    }
+  };
+  auto load_b = [&](int chunk) {
+#pragma unroll
+    for (int j = 0; j < PIECES; j++) {
+      int64_t off = (int64_t)chunk * (CH * 128) + bwithin[j] * 16;
+      if (off > row_bytes - 16) off = row_bytes - 16;             // pieces past k are never multiplied
+      breg[j] = *reinterpret_cast<const int4v*>(bsrc[j] - bwithin[j] * 16 + off);
+    }
+  };
+  auto multiply = [&](int set, int chunk) {
+    const uint8_t* sb = s_b[set];
+#pragma unroll
+    for (int u = 0; u < CH; u++) {
+      const int4v lo = *reinterpret_cast<const int4v*>(sb + u * NC * 128 + rd_lo);
+      const int4v hi = *reinterpret_cast<const int4v*>(sb + u * NC * 128 + rd_hi);
+      const int4v a = (int64_t)chunk * CH + u < npanels ? af[set][u] : int4v{0, 0, 0, 0};
+      const int8v bfrag = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      acc[u & 1] = mma16<T>::template run<0>(a, bfrag, acc[u & 1], idx[set][u]);
+    }
+  };
+  auto store_b = [&](int set) {
+#pragma unroll
+    for (int j = 0; j < PIECES; j++) *reinterpret_cast<int4v*>(s_b[set] + bdst[j]) = breg[j];
+  };
+  load_b(0);
+  load_a(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  // one barrier per chunk: a buffer is rewritten two iterations after it was read, and every wave
+  // passes the barrier in between only after that read
+  for (int ch = 0; ch < nchunks; ch += 2) {
+    store_b(0);
+    if (ch + 1 < nchunks) { load_b(ch + 1); load_a(1, ch + 1); }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    multiply(0, ch);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ch + 1 < nchunks) {
+      store_b(1);
+      if (ch + 2 < nchunks) { load_b(ch + 2); load_a(0, ch + 2); }
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      multiply(1, ch + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  if (!active || li >= n_dense) return;
+  const acc_t sum = acc[0] + acc[1];
+  const int64_t row = i0 + lk * 4;           // D layout: column l%16, rows 4*(l/16) + r
+  OutT o[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_value(sum[r], scale, bias, row + r, act));
+  if constexpr (C_JMAJOR) {
+    *reinterpret_cast<Pack<OutT, 4>*>(c + (int64_t)li * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; r++) c[(row + r) * ldc + li] = o[r];
+  }
+}
+
 template <typename T, typename OutT>
 int launch_narrow(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int64_t ldb, int64_t n_dense,
                   void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
   dim3 grid((unsigned)(n_sparse / 16));
-  // waves per block: one 16-row block per wave when that already gives two waves per CU, else split k
   const int64_t blocks = n_sparse / 16, npanels = k * (int64_t)sizeof(T) / 128;
-  int nwaves = blocks >= 512 ? 1 : kNarrowWaves;
+  if (blocks >= 512) {          // enough row blocks: several per workgroup, dense operand through LDS
+    const bool jm = c_layout == TF24_COL_MAJOR;
+    const int nw = blocks / 4 >= kNarrowSharedMin ? 4 : 2;      // four row blocks per workgroup only if that leaves enough workgroups
+    dim3 sgrid((unsigned)((blocks + nw - 1) / nw));
+    auto go = [&](auto jmajor, auto nc, auto nwc) {
+      hipLaunchKernelGGL((spmm_narrow_shared<T, OutT, decltype(jmajor)::value, decltype(nc)::value, decltype(nwc)::value>), sgrid,
+                         dim3(64 * decltype(nwc)::value), 0, s,
+                         (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                         (OutT*)c, ldc, (const OutT*)bias, scale, act);
+    };
+    auto go_nw = [&](auto jmajor, auto nc) {
+      if (nw == 4) go(jmajor, nc, std::integral_constant<int, 4>{}); else go(jmajor, nc, std::integral_constant<int, 2>{});
+    };
+    if (n_dense <= 8) { if (jm) go_nw(std::true_type{}, std::integral_constant<int, 8>{}); else go_nw(std::false_type{}, std::integral_constant<int, 8>{}); }
+    else { if (jm) go_nw(std::true_type{}, std::integral_constant<int, 16>{}); else go_nw(std::false_type{}, std::integral_constant<int, 16>{}); }
+    return check_launch("tf24_spmm");
+  }
+  int nwaves = kNarrowWaves;                 // few row blocks: the waves of a block split k
   while (nwaves > 1 && npanels / nwaves < 4) nwaves /= 2;
   if (c_layout == TF24_COL_MAJOR)
     hipLaunchKernelGGL((spmm_narrow<T, OutT, true>), grid, dim3(64 * nwaves), 0, s, (const uint8_t*)av, (const uint8_t*)am, n_sparse, k,
@@ -949,10 +1084,12 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
                    (n_dense <= MidCfg::BJ ||
                     (tile_cost<T, MidCfg>(n_sparse, k, n_dense, ws_bytes, 0.55).blocks <= 256 &&
                      tile_cost<T, MidCfg>(n_sparse, k, n_dense, ws_bytes, 0.55).us < tile_cost<T, TiledCfg>(n_sparse, k, n_dense, ws_bytes, 0.95).us));
-  // at most 8 dense columns: one pass over the compressed operand, no staging; up to 16 when the
-  // tiled kernel cannot cut k into pieces (no workspace), which it needs to fill the chip
+  // at most 8 dense columns: one pass over the compressed operand; up to 16 when the sparse operand
+  // has enough rows for the four-row-block form of that kernel (13.0 against 15.7 us on 11008 rows,
+  // but 19.7 against 18.6 us on 8192), or when the tiled kernel cannot cut k into pieces (no
+  // workspace), which it needs to fill the chip
   const bool narrow = panel && b_layout == TF24_ROW_MAJOR &&
-                      (n_dense <= 8 || (n_dense <= kNarrowMaxDense && !(slim && workspace)));
+                      (n_dense <= 8 || (n_dense <= kNarrowMaxDense && (n_sparse / 64 >= kNarrowSharedMin || !(slim && workspace))));
   if constexpr (std::is_same<T, i8_t>::value) {        // integer product: int32 accumulators, results and bias
     if (narrow) return launch_narrow<T, int32_t>(av, am, n_sparse, k, b, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
     if (slim) return launch_tiled<T, int32_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);

@@ -450,7 +450,7 @@ def main():
             "unit": "GB/s", "n_gpus": 1, "steps": 200, "warmup": 20, "ms_per_step": round(first["us"] / 1e3, 5),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "not a BASELINE config: tokens x W[11008,4096]^T, fp16, W 2:4 along K (decoding shapes)", "seed": 3},
-            "roofline": {"bound": "hbm", "kernel": "spmm_narrow (8 tokens)", "achieved": first["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "roofline": {"bound": "hbm", "kernel": "spmm_narrow_shared (8 tokens)", "achieved": first["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": first["frac_of_hbm_peak"], "traffic": None},
             "by_tokens": rows, "cpu_baseline": None}))
         return

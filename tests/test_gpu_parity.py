@@ -830,7 +830,7 @@ def test_spmm_narrow_dense_operand(cuda, dtype, m, k):
 @pytest.mark.parametrize("n,k", [(320, 1024), (8192, 1408 * 2)])
 def test_spmm_16_columns_without_workspace(cuda, dtype, n, k):
     """Through the C ABI with no workspace the tiled kernel cannot cut k into pieces, and 16 dense
-    columns take the one-pass kernel (four waves per block at 320 rows, one at 8192)."""
+    columns take the one-pass kernel (four waves that split k at 320 rows, the LDS-shared form at 8192)."""
     import sparse
     from sparse import _native as N
     m = 16
@@ -853,13 +853,15 @@ def test_spmm_16_columns_without_workspace(cuda, dtype, n, k):
     assert out.cpu().to(torch.float64).equal(ref.to(torch.float64))
 
 
+@pytest.mark.parametrize("n", [8192, 10272])
 @pytest.mark.parametrize("dtype", [F16, E4M3])
-def test_spmm_narrow_one_wave_per_block(cuda, dtype):
-    """Many sparse rows and few dense columns (16 through the tiled kernel's 64-wide tiles, 8 through the
-    one-pass kernel with one wave per 16-row block; fewer rows split k over four waves:
-    test_spmm_narrow_dense_operand); k not a multiple of the one-pass kernel's load batches."""
+def test_spmm_narrow_one_wave_per_block(cuda, dtype, n):
+    """Many sparse rows and few dense columns: the one-pass kernel whose waves own one 16-row block each
+    and share the dense operand through LDS (two blocks per workgroup at 8192 rows, four at 10272, where
+    the last workgroup has two idle waves and 16 columns also take this kernel; fewer rows split k over
+    four waves: test_spmm_narrow_dense_operand); k not a multiple of the 16-panel chunks."""
     import sparse
-    n, k, m = 8192, 1408 if dtype == F16 else 2816, 16
+    k, m = 1408 if dtype == F16 else 2816, 16
     w, x = _small_ints((n, k), 131, -2, 3).to(dtype), _small_ints((m, k), 132, -2, 3).to(dtype)
     mask = oracle.prune24_mask(w.float())
     ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
