@@ -853,15 +853,16 @@ def test_spmm_16_columns_without_workspace(cuda, dtype, n, k):
     assert out.cpu().to(torch.float64).equal(ref.to(torch.float64))
 
 
+@pytest.mark.parametrize("panels", [1, 17, 22])
 @pytest.mark.parametrize("n", [8192, 10272])
 @pytest.mark.parametrize("dtype", [F16, E4M3])
-def test_spmm_narrow_one_wave_per_block(cuda, dtype, n):
+def test_spmm_narrow_one_wave_per_block(cuda, dtype, n, panels):
     """Many sparse rows and few dense columns: the one-pass kernel whose waves own one 16-row block each
     and share the dense operand through LDS (two blocks per workgroup at 8192 rows, four at 10272, where
     the last workgroup has two idle waves and 16 columns also take this kernel; fewer rows split k over
     four waves: test_spmm_narrow_dense_operand); k not a multiple of the 16-panel chunks."""
     import sparse
-    k, m = 1408 if dtype == F16 else 2816, 16
+    k, m = panels * (64 if dtype == F16 else 128), 16      # 1 panel, one chunk + 1, 22 panels
     w, x = _small_ints((n, k), 131, -2, 3).to(dtype), _small_ints((m, k), 132, -2, 3).to(dtype)
     mask = oracle.prune24_mask(w.float())
     ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
