@@ -389,3 +389,44 @@ def test_adamw_step_optimizer_phases(cuda):
     assert opt.t == 6 and len(opt.sliding_window) == 2                    # the window stops growing after the switch
     with pytest.raises(ValueError):
         sparse.AdamW_STEP([w], option=3)
+
+
+def test_entry_points_under_graph_capture(cuda):
+    """The library only launches kernels on the stream it is given (no allocation, no synchronisation,
+    no memset), so its calls can be recorded into a HIP graph: compression, both matmul forms (the
+    split one with its workspace and reduction) and the masked decay are captured once and replayed
+    on new contents of the same buffers, with eager work between the replays; every replay must give
+    the bits of the eager calls."""
+    import sparse
+    n, k, m = 512, 4096, 48
+    gen = torch.Generator().manual_seed(71)
+    w = torch.randn(n, k, generator=gen).half().to(cuda)
+    x = torch.randn(m, k, generator=gen).half().to(cuda)
+    g32 = torch.randn(n, k, generator=gen).to(cuda)
+
+    def work():
+        s = sparse.to_sparse_semi_structured(w)                     # magnitude rule: no random numbers
+        y = torch.mm(x, s.t())                                      # few dense columns: k pieces + reduction
+        z = torch.mm(s, w.t())                                      # [n, n]: k-strided dense operand
+        grad = g32.clone()
+        sparse.masked_add_(grad, w.float(), (s.to_dense() != 0), alpha=2e-4)
+        return y, z, grad
+
+    work()                                                          # warm up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            captured = work()
+    torch.cuda.synchronize()
+    for it in range(3):
+        w.copy_(torch.randn(n, k, generator=gen).half())
+        x.copy_(torch.randn(m, k, generator=gen).half())
+        g32.copy_(torch.randn(n, k, generator=gen))
+        eager = [t.clone() for t in work()]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("x @ S.t", "S @ w.t", "masked decay"), captured, eager):
+            assert torch.equal(a, b), (it, name)
