@@ -342,8 +342,8 @@ def fp8_workload(steps, warmup):
 
 
 def decode_workload(iters=200):
-    """Not a BASELINE config: a few tokens against the config-3 weight (W[11008,4096] fp16, 2:4 along K), the
-    shape of decoding with a compressed weight.  Bound by one pass over the compressed operand (values +
+    """Not a BASELINE config: 8 to 1024 tokens against the config-3 weight (W[11008,4096] fp16, 2:4 along K), the
+    shapes of decoding and of small batches with a compressed weight.  Bound by one pass over the compressed operand (values +
     metadata = 1.125 bytes per dense weight element).  Direct C-ABI launches on preallocated buffers;
     returns one row per token count with the dense hipBLASLt time on the decompressed weight beside it."""
     import sparse
@@ -357,7 +357,7 @@ def decode_workload(iters=200):
     Wd_t = S.to_dense().t()
     v, mt, st = S._store_values, S._store_meta, N.stream_ptr()
     rows = []
-    for tokens in (8, 16, 32, 64, 128):
+    for tokens in (8, 16, 32, 64, 128, 256, 512, 1024):
         x = torch.randn(tokens, K, generator=gen).half().to(dev)
         out = torch.empty(tokens, Nw, dtype=torch.float16, device=dev)
         wsb = lib.tf24_spmm_workspace_bytes(N.F16, Nw, K, tokens)
@@ -417,7 +417,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=["spmm", "train", "fp8", "decode"], default="spmm",
                     help="spmm: BASELINE configs[2] (default, the judged line); train: configs[3] MLP training step; "
-                         "fp8: configs[4] e4m3 MVUE + spMM; decode: 8-128 tokens against the config-3 weight (not a BASELINE config)")
+                         "fp8: configs[4] e4m3 MVUE + spMM; decode: 8-1024 tokens against the config-3 weight (not a BASELINE config)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-convert", action="store_true", help="skip the conversion-kernel table")
     a = ap.parse_args()
