@@ -1159,7 +1159,9 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
   const int64_t bext = b_layout == TF24_ROW_MAJOR ? k : n_dense;
   if (ldb < bext || ldb % dmult) return fail(TF24_ERR_STRIDE, "%s: ldb %lld must be >= %lld and a multiple of %lld", fn, (long long)ldb, (long long)bext, (long long)dmult);
   const int64_t cext = c_layout == TF24_ROW_MAJOR ? n_dense : n_sparse;
-  if (ldc < cext || ldc % 4) return fail(TF24_ERR_STRIDE, "%s: ldc %lld must be >= %lld and a multiple of 4", fn, (long long)ldc, (long long)cext);
+  // rows of the output leave as 16-byte stores: 8 elements of a 16-bit type, 4 of a 32-bit one
+  const int64_t cmult = (out_dtype == TF24_F16 || out_dtype == TF24_BF16) ? 8 : 4;
+  if (ldc < cext || ldc % cmult) return fail(TF24_ERR_STRIDE, "%s: ldc %lld must be >= %lld and a multiple of %lld", fn, (long long)ldc, (long long)cext, (long long)cmult);
   if (activation < TF24_ACT_NONE || activation > TF24_ACT_GELU) return fail(TF24_ERR_ARG, "%s: bad activation %d", fn, activation);
   return TF24_OK;
 }

@@ -11,7 +11,8 @@ from .decay import masked_add_
 from .adamw import MaskedDecayAdamW
 from .adamw_step import AdamW_STEP
 from .dense_ops import (soft_threshold24, sparse24, MVUE24_approx,
-                        soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton)
+                        soft_threshold24_triton, sparse24_triton, MVUE24_approx_triton,
+                        soft_threshold24_torch, sparse24_torch, MVUE24_approx_torch)
 from .sparse_linear_transpose import SparseLinearTranspose, sparse_linear_transpose
 from .sparse_semi_structured_linear import sparse_semi_structured_linear
 from .GELUglu import GELUglu, gelu_glu
@@ -24,6 +25,7 @@ __all__ = [
     "masked_add_", "MaskedDecayAdamW", "AdamW_STEP",
     "soft_threshold24", "sparse24", "MVUE24_approx",
     "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
+    "soft_threshold24_torch", "sparse24_torch", "MVUE24_approx_torch",
     "SparseLinearTranspose", "sparse_linear_transpose",
     "sparse_semi_structured_linear",
     "GELUglu", "gelu_glu",

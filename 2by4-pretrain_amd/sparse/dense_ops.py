@@ -6,13 +6,19 @@
 
 Outputs have the input's shape, dtype and strides; the mask is returned in the dense dtype
 (1.0 / 0.0), as the reference does.  The reference's `*_triton` names are kept as aliases.
+
+The reference's `*_torch` forms (sparse/legacy.py:26-40, :96-117, :227-268: the same three operators
+written with argsort / multinomial over the flattened tensor, any shape, int32 mask) are kept as
+names on top of the same kernels: the tensor is viewed as rows of its last dimension, groups of 4
+run along the flattened storage exactly as `reshape(group, 4)` cuts them.
 """
 import torch
 
 from . import _native as N
 
 __all__ = ["soft_threshold24", "sparse24", "MVUE24_approx",
-           "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton"]
+           "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",
+           "soft_threshold24_torch", "sparse24_torch", "MVUE24_approx_torch"]
 
 
 def _prepare(dense):
@@ -64,3 +70,33 @@ def MVUE24_approx(dense, rand=None):
 soft_threshold24_triton = soft_threshold24
 sparse24_triton = sparse24
 MVUE24_approx_triton = MVUE24_approx
+
+
+def _as_rows(weight):
+    """Contiguous 2-d view [rows, cols] of a tensor of any shape whose groups of 4 along the flattened
+    storage are the groups of 4 along cols."""
+    if weight.numel() % 8:
+        raise RuntimeError(f"number of elements {weight.numel()} must be a multiple of 8")
+    flat = weight.contiguous()
+    cols = flat.shape[-1] if flat.dim() >= 2 and flat.shape[-1] % 8 == 0 else 8
+    return flat.view(-1, cols)
+
+
+def sparse24_torch(weight):
+    """legacy.py:26-40: (weight * mask, mask) with an int32 mask of weight's shape."""
+    sparse, mask = sparse24(_as_rows(weight))
+    return sparse.view(weight.shape), mask.view(weight.shape).to(torch.int32)
+
+
+def soft_threshold24_torch(weight):
+    """legacy.py:96-117: (soft-thresholded weight, int32 mask)."""
+    sparse, mask = soft_threshold24(_as_rows(weight))
+    return sparse.view(weight.shape), mask.view(weight.shape).to(torch.int32)
+
+
+def MVUE24_approx_torch(weight, rand=None):
+    """legacy.py:227-268: the MVUE24 estimate of weight, same shape."""
+    rows = _as_rows(weight)
+    if rand is not None:
+        rand = rand.contiguous().view(rows.shape)
+    return MVUE24_approx(rows, rand).view(weight.shape)

@@ -50,9 +50,13 @@ class sparse_linear_transpose(autograd.Function):
         input, weight_T, bias = ctx.saved_tensors
         grad_input = grad_weight = grad_bias = None
         with torch.autocast(device_type="cuda", enabled=False):
-            if grad_output.stride() == (0,) * grad_output.dim():       # expanded scalar gradient
-                grad_output = torch.ones_like(grad_output)
+            # An expanded scalar gradient (all strides 0: the layer's output fed straight into .sum() or
+            # .mean()) is materialised with its values.  The reference replaces a 3-d one by ones
+            # (README.md:186-187), which is the same thing after .sum() and scales every gradient by the
+            # element count after .mean(); the values are kept here.
             grad_output = grad_output.reshape(-1, grad_output.shape[-1])
+            if grad_output.stride(-1) != 1 or grad_output.stride(0) < grad_output.shape[-1]:
+                grad_output = grad_output.contiguous()
             if grad_output.dtype != input.dtype:
                 grad_output = grad_output.to(input.dtype)
             if ctx.needs_input_grad[0]:

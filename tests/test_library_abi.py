@@ -92,6 +92,8 @@ def test_transposable_and_spmm_validators(native):
     assert sp(N.E4M3, 32, 64, 16) == -1 and sp(N.E4M3, 32, 128, 8) == -1
     assert sp(N.F32, 32, 64, 8) == -2 and sp(N.F16, 32, 64, 8, out=N.E4M3) == -2
     assert sp(N.F16, 32, 64, 8, ldb=32) == -3 and sp(N.F16, 32, 64, 8, ldc=16) == -3
+    # output rows leave as 16-byte segments: ldc % 8 for 16-bit results, % 4 for 32-bit ones
+    assert sp(N.F16, 32, 64, 8, ldc=36) == -3 and sp(N.F16, 32, 64, 8, ldc=40) == 0 and sp(N.F16, 32, 64, 8, ldc=36, out=N.F32) == 0
     assert sp(N.F16, 32, 64, 8, act=5) == -5 and sp(N.F16, 32, 64, 8, bl=3) == -5
 
 
