@@ -7,6 +7,7 @@
 // live entirely in its registers), a 256-lane block covers 8R rows x 128 columns, and the
 // compressed tile is transposed through LDS so that values and metadata leave row-major with
 // full-line stores.
+#include <mutex>
 #include <type_traits>
 
 #include "tf24_common.hpp"
@@ -459,6 +460,64 @@ extern "C" int tf24_prune_compress_rowsum(const void* dense, int in_dtype, int l
     default: hipLaunchKernelGGL((rowsum_finish<bf16_t>), grid, dim3(kThreads), 0, s, (const float*)workspace, nblocks, m, (bf16_t*)rowsum); break;
   }
   return check_launch(fn);
+}
+
+// ------------------------------------------------------------------------------------------
+// tf24_prune_compress_rowsum without a caller workspace: the partial row sums go to a fixed array in
+// the library's own device image.  Each GPU the library runs on holds its own copy of the array (at
+// its own address) until the process ends.
+// ------------------------------------------------------------------------------------------
+namespace tf24 {
+namespace {
+
+constexpr int64_t kRowsumScratchFloats = (int64_t)1 << 20;          // 4 MiB: m * ceil(k / 128) <= 2^20
+static __device__ __align__(256) float scratch[kRowsumScratchFloats];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices];                                   // device address of `scratch`, per device
+
+// Device address of `scratch` on the current device (looked up once per device; in host code the
+// array's name is only a handle for this lookup, never a device address).
+int scratch_address(const char* fn, float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(TF24_ERR_LAUNCH, "%s: cannot identify the current device (%d)", fn, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(TF24_ERR_LAUNCH, "%s: hipGetSymbolAddress failed: %s", fn, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return TF24_OK;
+}
+
+}  // namespace
+}  // namespace tf24
+
+extern "C" int64_t tf24_prune_compress_rowsum_static_max_bytes(void) {
+  return tf24::kRowsumScratchFloats * (int64_t)sizeof(float);
+}
+
+extern "C" int tf24_prune_compress_rowsum_static(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                                                 int mode, const void* mask, int mask_dtype, int64_t mask_ld,
+                                                 const float* rnd, int64_t rand_ld,
+                                                 void* values, int out_dtype, void* meta, int out_layout,
+                                                 void* rowsum, int rowsum_dtype, void* stream) {
+  using namespace tf24;
+  const char* fn = "tf24_prune_compress_rowsum_static";
+  const int64_t need = tf24_prune_compress_rowsum_workspace_bytes(m, k);
+  if (need > tf24_prune_compress_rowsum_static_max_bytes())
+    return fail(TF24_ERR_SHAPE, "%s: a %lld x %lld matrix needs %lld bytes of partial sums, the built-in scratch holds %lld "
+                "(m * ceil(k / 128) <= %lld); use tf24_prune_compress_rowsum with a workspace", fn, (long long)m, (long long)k,
+                (long long)need, (long long)tf24_prune_compress_rowsum_static_max_bytes(), (long long)kRowsumScratchFloats);
+  float* ptr = nullptr;
+  if (int rc = scratch_address(fn, &ptr)) return rc;
+  // every partial sum the second kernel reads is written by the first one: nothing has to start at zero
+  return tf24_prune_compress_rowsum(dense, in_dtype, layout, ld, m, k, mode, mask, mask_dtype, mask_ld, rnd, rand_ld, values, out_dtype,
+                                    meta, out_layout, rowsum, rowsum_dtype, ptr, tf24_prune_compress_rowsum_static_max_bytes(), stream);
 }
 
 namespace tf24 {

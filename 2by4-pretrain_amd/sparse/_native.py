@@ -37,6 +37,8 @@ _SIGNATURES = {
     "tf24_mvue_uniforms": (_i, [ctypes.c_uint64, ctypes.c_uint64, _i64, _i64, _i, _p, _i64, _p]),
     "tf24_prune_compress_rowsum": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p, _i, _p, _i64, _p]),
     "tf24_prune_compress_rowsum_workspace_bytes": (_i64, [_i64, _i64]),
+    "tf24_prune_compress_rowsum_static": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _i, _i64, _p, _i64, _p, _i, _p, _i, _p, _i, _p]),
+    "tf24_prune_compress_rowsum_static_max_bytes": (_i64, []),
     "tf24_prune_compress_dual": (_i, [_p, _i, _i64, _i64, _i64, _p, _i, _i64, _p, _p, _p, _p, _i, _i, _p]),
     "tf24_prune_compress_dual_validate": (_i, [_i, _i64, _i64, _i64, _i, _i64, _i, _i]),
     "tf24_decompress": (_i, [_p, _i, _p, _i, _i64, _i64, _p, _p]),

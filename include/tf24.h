@@ -135,6 +135,25 @@ int tf24_prune_compress_rowsum(const void* dense, int in_dtype, int layout, int6
 int64_t tf24_prune_compress_rowsum_workspace_bytes(int64_t m, int64_t k);
 
 /*
+ * tf24_prune_compress_rowsum for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and so cannot bring a workspace.  No counterpart in
+ * the reference.  Same arguments and bit-identical results; the partial row sums go to a fixed 4 MiB
+ * array inside the library's device image instead (tf24_prune_compress_rowsum_static_max_bytes()), which
+ * every GPU the library runs on holds until the process ends.  The call allocates and frees nothing.
+ *   limit   tf24_prune_compress_rowsum_workspace_bytes(m, k) <= 4 MiB, i.e. m * ceil(k / 128) <= 2^20
+ *           (config 4's 3072 x 12288 gradient needs 1.2 MiB); larger shapes return TF24_ERR_SHAPE.
+ *   sharing every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different
+ *           streams, or threads on the same device) race on it and must be serialised by the caller.
+ *           Nothing in the array has to start at zero: each call writes every partial sum it reads.
+ */
+int tf24_prune_compress_rowsum_static(const void* dense, int in_dtype, int layout, int64_t ld, int64_t m, int64_t k,
+                                      int mode, const void* mask, int mask_dtype, int64_t mask_ld,
+                                      const float* rand, int64_t rand_ld,
+                                      void* values, int out_dtype, void* meta, int out_layout,
+                                      void* rowsum, int rowsum_dtype, void* stream);
+int64_t tf24_prune_compress_rowsum_static_max_bytes(void);
+
+/*
  * Mask-driven 2:4 compression of W and of W^T from ONE read of W and of the mask:
  *   (values, meta)      = tf24_prune_compress(W   [m,k] row-major,          mode MASK, mask)
  *   (values_t, meta_t)  = tf24_prune_compress(W^T [k,m] (W read by columns), mode MASK, mask^T)
