@@ -1,13 +1,14 @@
 """Benchmark of the 2:4 sparse hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|train|fp8] [--no-cpu] [--no-convert]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|train|fp8|decode|traffic] [--no-cpu] [--no-convert] [--no-extra]
 
 Default workload: BASELINE config 3 -- fp16 2:4 spMM forward  Y[8192,11008] = X[8192,4096] . W^T
 (W[11008,4096] magnitude-pruned along K) plus the transposed product dX[8192,4096] = dY . W with
 the transposable-masked W compressed along its other axis.  One "step" = those two matmuls.
 Prints ONE JSON line: whole-step throughput, the dominant kernel's roofline (HIP-event timed in
 the same region), the dense hipBLASLt GEMM on the same shapes, per-kernel GB/s of the conversion
-kernels at BASELINE config 2 sizes, and the CPU oracle timed on a bounded sample.
+kernels at BASELINE config 2 sizes, the fp8 product of configs[4] and the training step of configs[3]
+with their dense comparators, and the CPU oracle timed on a bounded sample.
 """
 import argparse
 import json
@@ -24,10 +25,18 @@ import torch  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_DENSE_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA; SMFMAC executes MACs at this rate
-# HBM bytes per spmm launch (mean of forward and transposed) from two rocprofv3 --pmc runs of this file:
-# FETCH_SIZE 424831 KiB + WRITE_SIZE 120846 KiB, both counters reading factor 1.00 on a copy kernel of known size
-SPMM_TRAFFIC_BYTES = (424831 + 120846) * 1024
-
+MFMA_DENSE_PEAK_FP8_TFLOPS = 5000.0
+# Bytes that cross the L2 <-> memory-fabric boundary per spmm launch of config 3 (mean of forward and
+# transposed), from two `rocprofv3 --pmc` runs of `bench.py --workload traffic` (FETCH_SIZE, then
+# WRITE_SIZE; KiB per dispatch), each scaled by known / counted bytes of a plain 128 MiB device copy in
+# the same run: FETCH_SIZE 414876 KiB x 2.00 (the counter books this GPU's 128-byte read requests as 64
+# bytes: every streaming kernel of known footprint reads 0.50 of its bytes, and the 32-byte-unit request
+# counter TCC_EA0_RDREQ_DRAM_32B gives the same 848 MB), WRITE_SIZE 120837 KiB x 1.00.  The infinity
+# cache sits behind this boundary, so part of it never reaches HBM.  A profiled constant, not
+# something this run measures: emitted for the config-3 shape only, with its source.
+SPMM_TRAFFIC_PROFILED = int(414876 * 1024 * 2.0 + 120837 * 1024 * 1.0)
+SPMM_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over `bench.py --workload traffic`, factors 2.00 / 1.00 from the "
+                       "128 MiB device copy of the same runs; L2 <-> fabric bytes (infinity cache behind it); summary under profiles/")
 
 def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -50,25 +59,34 @@ def settle(fn, seconds=SETTLE_S):
         torch.cuda.synchronize()
 
 
-def time_rotating(fn, nsets, iters, warmup):
-    """Average device time per call (microseconds) of fn(i % nsets), HIP events on the current stream."""
+def time_rotating(fn, nsets, iters, warmup, batch=10):
+    """Device time per call of fn(i % nsets) in microseconds, HIP events on the current stream: `iters`
+    timed launches in batches of `batch` back-to-back launches (an event pair around every single
+    launch would put the launch latency of each kernel inside its own interval).  Returns the
+    median, the mean, the fastest and the slowest of the batch means."""
     settle(lambda i: fn(i % nsets))
     for i in range(warmup):
         fn(i % nsets)
-    start, end = _events(2)
+    nb = max(1, (iters + batch - 1) // batch)
+    ev = _events(nb + 1)
     torch.cuda.synchronize()
-    start.record()
-    for i in range(iters):
-        fn(i % nsets)
-    end.record()
+    i = 0
+    ev[0].record()
+    for b in range(nb):
+        for _ in range(batch):
+            fn(i % nsets); i += 1
+        ev[b + 1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(end) * 1e3 / iters
+    per = sorted(ev[b].elapsed_time(ev[b + 1]) * 1e3 / batch for b in range(nb))
+    return {"median": per[len(per) // 2] if len(per) % 2 else 0.5 * (per[len(per) // 2 - 1] + per[len(per) // 2]),
+            "mean": sum(per) / len(per), "min": per[0], "max": per[-1], "launches": nb * batch}
 
 
 # --------------------------------------------------------------------------------------------
-def conversion_kernels(iters=40, warmup=8, nsets=4):
+def conversion_kernels(iters=100, warmup=16, nsets=8):
     """BASELINE config 2: W[8192,8192] bf16 ~ N(0,1) seed 1; direct C-ABI launches on preallocated
-    buffers, inputs rotated over `nsets` buffer sets so the 256 MB last-level cache cannot serve them."""
+    buffers, inputs and outputs rotated over `nsets` buffer sets (8 x 128 MiB of the smallest input,
+    8 x 256 MiB of the float32 ones) so that the 256 MB last-level cache cannot serve repeats."""
     from sparse import _native as N
     lib = N.lib()
     dev = torch.device("cuda:0")
@@ -112,13 +130,13 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
         N.check(lib.tf24_prune_compress(P[i].data_ptr(), N.F32, N.ROW_MAJOR, k, m, k, N.PRUNE_MASK, bmask[i].data_ptr(), N.U8, k,
                                         None, 0, values[i].data_ptr(), N.F16, meta[i].data_ptr(), N.COMPRESSED_PANEL, st))
 
-    values_t = [torch.empty(k, m // 2, dtype=torch.float16, device=dev) for _ in range(2)]
-    meta_t = [torch.empty(k, m // 16, dtype=torch.int16, device=dev) for _ in range(2)]
+    values_t = [torch.empty(k, m // 2, dtype=torch.float16, device=dev) for _ in range(nsets)]
+    meta_t = [torch.empty(k, m // 16, dtype=torch.int16, device=dev) for _ in range(nsets)]
 
     def mask_compress_pair(i):
         N.check(lib.tf24_prune_compress_dual(P[i].data_ptr(), N.F32, k, m, k, bmask[i].data_ptr(), N.U8, k,
-                                             values[i].data_ptr(), meta[i].data_ptr(), values_t[i % 2].data_ptr(),
-                                             meta_t[i % 2].data_ptr(), N.F16, N.COMPRESSED_PANEL, st))
+                                             values[i].data_ptr(), meta[i].data_ptr(), values_t[i].data_ptr(),
+                                             meta_t[i].data_ptr(), N.F16, N.COMPRESSED_PANEL, st))
 
     def copy(i):
         sp[i].copy_(W[i])
@@ -141,10 +159,12 @@ def conversion_kernels(iters=40, warmup=8, nsets=4):
     for i in range(nsets):
         transposable(i)     # masks for the decay / mask-compress legs
     for name, fn, nbytes in table:
-        us = time_rotating(fn, nsets, iters, warmup)
+        t = time_rotating(fn, nsets, iters, warmup)
+        us = t["median"]
         gbps = nbytes / us / 1e3
-        out.append({"kernel": name, "us": round(us, 2), "bytes": nbytes, "GBps": round(gbps, 1),
-                    "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)})
+        out.append({"kernel": name, "us": round(us, 2), "us_mean": round(t["mean"], 2), "us_min": round(t["min"], 2),
+                    "us_max": round(t["max"], 2), "launches": t["launches"], "buffer_sets": nsets, "bytes": nbytes,
+                    "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)})
     return out
 
 
@@ -223,6 +243,9 @@ def train_workload(steps, warmup):
     tokens, d, h = 12 * 1024, 768, 3072
     x = torch.randn(tokens, d, device=dev)
     target = torch.randn(tokens, d, device=dev)
+    # a mean over 12288 x 768 outputs puts dY near 1e-7, below fp16's normal range: fixed loss scale
+    # (a power of two), gradients unscaled in one multi-tensor launch, in both models
+    loss_scale = 4096.0
 
     def build(kind):
         torch.manual_seed(2)
@@ -248,7 +271,8 @@ def train_workload(steps, warmup):
                     out = proj(F.gelu(fc(x)))
             loss = F.mse_loss(out.float(), target)
             opt.zero_grad(set_to_none=True)
-            loss.backward()
+            (loss * loss_scale).backward()
+            torch._foreach_mul_([p.grad for p in params], 1.0 / loss_scale)
             if kind == "sparse":
                 with torch.no_grad():
                     for p in params:
@@ -369,10 +393,10 @@ def decode_workload(iters=200):
 
         def dense_mm(_i):
             torch.mm(x, Wd_t, out=out)
-        us = time_rotating(sparse_mm, 1, iters, 20)
+        us = time_rotating(sparse_mm, 1, iters, 20)["median"]
         ref = x.float() @ Wd_t.float()
         rel = ((out.float() - ref).norm() / ref.norm()).item()
-        dus = time_rotating(dense_mm, 1, iters, 20)
+        dus = time_rotating(dense_mm, 1, iters, 20)["median"]
         nbytes = Nw * K * 9 // 8 + tokens * K * 2 + tokens * Nw * 2
         rows.append({"tokens": tokens, "us": round(us, 2), "dense_hipblaslt_us": round(dus, 2), "speedup_vs_dense": round(dus / us, 3),
                      "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
@@ -382,7 +406,8 @@ def decode_workload(iters=200):
 
 def cpu_baseline_spmm(threads):
     """The oracle (pure-PyTorch port of the reference semantics) on the host cores, on config 3 itself:
-    prune+compress and transposable mask of W, then both dense masked fp32 products once."""
+    prune+compress and transposable mask of W, then both dense masked fp32 products; one warm-up
+    repetition and three timed ones, the median reported."""
     import oracle
     torch.set_num_threads(threads)
     gen = torch.Generator().manual_seed(3)
@@ -390,24 +415,97 @@ def cpu_baseline_spmm(threads):
     X = torch.randn(M, K, generator=gen).half()
     W = (0.02 * torch.randn(Nw, K, generator=gen)).half()
     dY = torch.randn(M, Nw, generator=gen).half()
-    t0 = time.perf_counter()
+
+    def timed(fn, reps=3):
+        fn()                                             # warm-up
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2]
+
     mask = oracle.prune24_mask(W)
-    oracle.compress24(W, mask=mask)
-    t_conv = time.perf_counter() - t0
-    t0 = time.perf_counter()
     w_t, _ = oracle.transposable_mask(W)
-    t_tr = time.perf_counter() - t0
     Wm = torch.where(mask, W, torch.zeros_like(W))
-    oracle.spmm_ref(X[:64], Wm)
-    t0 = time.perf_counter()
-    oracle.spmm_ref(X, Wm)
-    oracle.spmm_ref(dY, w_t.t().contiguous())
-    t_mm = time.perf_counter() - t0
+    Wt = w_t.t().contiguous()
+    t_conv = timed(lambda: oracle.compress24(W, mask=oracle.prune24_mask(W)))
+    t_tr = timed(lambda: oracle.transposable_mask(W))
+    t_mm = timed(lambda: (oracle.spmm_ref(X, Wm), oracle.spmm_ref(dY, Wt)))
     tflops = 2 * 2.0 * M * Nw * K / t_mm / 1e12
     return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"the whole of config 3 once: oracle.spmm_ref fp32 forward + transposed ({t_mm:.2f} s); "
+            "sample": f"the whole of config 3, 1 warm-up + 3 timed repetitions, median: oracle.spmm_ref fp32 forward + transposed ({t_mm:.2f} s); "
                       f"oracle prune+compress of W {t_conv:.2f} s ({3.125 * Nw * K / t_conv / 1e9:.2f} GB/s algorithmic), "
                       f"oracle transposable mask of W {t_tr:.2f} s ({5.0 * Nw * K / t_tr / 1e9:.2f} GB/s algorithmic)"}
+
+
+def host_threads():
+    """Threads for the CPU leg: what the host gives this process (its affinity mask, and the
+    OMP_NUM_THREADS the box sets), not the machine's core count."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit() and int(env) > 0:
+        n = min(n, int(env))
+    return max(1, n)
+
+
+def traffic_workload(reps=8):
+    """Kernels of known footprint, then the config-3 products, each launched `reps` times on rotated
+    buffers: the workload of the `rocprofv3 --pmc` runs that calibrate the L2 <-> fabric byte counters
+    (counted / known bytes on the streaming kernels) and size the matmul's traffic with them."""
+    import sparse
+    from sparse import _native as N
+    lib = N.lib()
+    dev = torch.device("cuda:0")
+    m = k = 8192
+    n = m * k
+    nsets = 8
+    gen = torch.Generator(device=dev).manual_seed(1)
+    W = [torch.randn(m, k, device=dev, generator=gen).bfloat16() for _ in range(nsets)]
+    G = [1e-3 * torch.randn(m, k, device=dev, generator=gen) for _ in range(nsets)]
+    P = [torch.randn(m, k, device=dev, generator=gen) for _ in range(nsets)]
+    bmask = [torch.rand(m, k, device=dev, generator=gen) < 0.5 for _ in range(nsets)]
+    values = [torch.empty(m, k // 2, dtype=torch.float16, device=dev) for _ in range(nsets)]
+    meta = [torch.empty(m, k // 16, dtype=torch.int16, device=dev) for _ in range(nsets)]
+    dense = [torch.empty(m, k, dtype=torch.float16, device=dev) for _ in range(nsets)]
+    st = N.stream_ptr()
+    known = {}
+    for i in range(reps):
+        j = i % nsets
+        N.check(lib.tf24_masked_add(G[j].data_ptr(), N.F32, P[j].data_ptr(), N.F32, bmask[j].data_ptr(), N.U8, n, 2e-4, st))
+    known["masked_add_vec"] = {"read": 9 * n, "written": 4 * n}
+    for i in range(reps):
+        j = i % nsets
+        N.check(lib.tf24_prune_compress(W[j].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MAGNITUDE, None, N.U8, 0,
+                                        None, 0, values[j].data_ptr(), N.F16, meta[j].data_ptr(), N.COMPRESSED_PANEL, st))
+    known["prune_compress_row"] = {"read": 2 * n, "written": n + n // 8}
+    for i in range(reps):
+        j = i % nsets
+        N.check(lib.tf24_decompress(values[j].data_ptr(), N.F16, meta[j].data_ptr(), N.COMPRESSED_PANEL, m, k, dense[j].data_ptr(), st))
+    known["decompress_kernel"] = {"read": n + n // 8, "written": 2 * n}
+    for i in range(reps):
+        j = i % nsets
+        dense[j].view(torch.bfloat16).copy_(W[(j + 1) % nsets])
+    known["torch copy (bf16, 8192 x 8192)"] = {"read": 2 * n, "written": 2 * n}
+    torch.cuda.synchronize()
+    del W, G, P, bmask, values, meta, dense
+    M, K, Nw = 8192, 4096, 11008
+    g = torch.Generator().manual_seed(3)
+    X = torch.randn(M, K, generator=g).half().to(dev)
+    Wt = (0.02 * torch.randn(Nw, K, generator=g)).half().to(dev)
+    dY = torch.randn(M, Nw, generator=g).half().to(dev)
+    w_fwd = sparse.to_sparse_semi_structured(Wt)
+    _, tmask = sparse.TransposableSparse()(Wt)
+    w_bwd = sparse.to_sparse_semi_structured(Wt.T, mask=tmask.T)
+    for _ in range(reps):
+        torch.mm(X, w_fwd.t())
+        torch.mm(dY, w_bwd.t())
+    torch.cuda.synchronize()
+    known["spmm_pipe (config 3, per launch, algorithmic)"] = {"read": M * K * 2 + Nw * K * 9 // 8, "written": M * Nw * 2}
+    return {"launches_per_kernel": reps, "buffer_sets": nsets, "known_bytes_per_launch": known}
 
 
 def main():
@@ -415,11 +513,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["spmm", "train", "fp8", "decode"], default="spmm",
+    ap.add_argument("--workload", choices=["spmm", "train", "fp8", "decode", "traffic"], default="spmm",
                     help="spmm: BASELINE configs[2] (default, the judged line); train: configs[3] MLP training step; "
-                         "fp8: configs[4] e4m3 MVUE + spMM; decode: 8-1024 tokens against the config-3 weight (not a BASELINE config)")
+                         "fp8: configs[4] e4m3 MVUE + spMM; decode: 8-1024 tokens against the config-3 weight (not a BASELINE config); "
+                         "traffic: kernels of known footprint + the config-3 products, for rocprofv3 --pmc byte-counter runs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-convert", action="store_true", help="skip the conversion-kernel table")
+    ap.add_argument("--no-extra", action="store_true", help="skip the fp8 (configs[4]) and training-step (configs[3]) legs of the default line")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the 2:4 path has no multi-GPU component (--gpus must be 1)", file=sys.stderr)
@@ -428,6 +528,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+
+    if a.workload == "traffic":
+        print(json.dumps(traffic_workload()))
+        return
 
     if a.workload == "train":
         sparse_ms, dense_ms, sl, dl, flops, one_pass_ms = train_workload(a.steps, a.warmup)
@@ -484,8 +588,9 @@ def main():
                    "M": M, "K": K, "N": Nw, "seed": 3},
         "roofline": {"bound": "mfma", "kernel": "spmm (SMFMAC)", "achieved": round(executed_tflops, 2),
                      "peak": MFMA_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(executed_tflops / MFMA_DENSE_PEAK_TFLOPS, 4),
-                     "traffic": SPMM_TRAFFIC_BYTES,
-                     "algorithmic_bytes": 2 * (M * K + Nw * K // 2 + Nw * K // 16 + M * Nw),
+                     "traffic": SPMM_TRAFFIC_PROFILED,
+                     "traffic_source": SPMM_TRAFFIC_SOURCE,
+                     "algorithmic_bytes": M * K * 2 + Nw * K * 9 // 8 + M * Nw * 2,
                      "note": "achieved = executed flops (M*N*K, half the dense-equivalent 2MNK) per launch / HIP-event "
                              "launch time; SMFMAC executes MACs at the dense MFMA rate, so frac also equals "
                              "dense-equivalent rate / (2 x dense peak)",
@@ -496,10 +601,33 @@ def main():
         "speedup_vs_dense_gemm": round((dfwd_ms + dbwd_ms) / (fwd_ms + bwd_ms), 3),
         "rel_err_vs_dense_fp32": {"fwd": rel_f, "transposed": rel_b},
     }
+    if not a.no_extra:
+        # the other two single-GPU configs of the baseline, in the same line (each also runs alone
+        # with --workload fp8 / train)
+        torch.cuda.empty_cache()
+        step_ms, mm_ms, dense_ms, rel, f8 = fp8_workload(a.steps, a.warmup)
+        ex8 = (f8 / 2) / (mm_ms * 1e-3) / 1e12
+        line["fp8_config5"] = {
+            "workload": "BASELINE configs[4]: e4m3 A[16384,8192] x MVUE24-pruned B[8192,8192]^T, fp32 accumulate, bf16 out",
+            "spmm_ms": round(mm_ms, 4), "tflops_dense_equivalent": round(f8 / (mm_ms * 1e-3) / 1e12, 1),
+            "roofline_frac": round(ex8 / MFMA_DENSE_PEAK_FP8_TFLOPS, 4),
+            "dense_fp8_gemm_ms": None if dense_ms is None else round(dense_ms, 4),
+            "speedup_vs_dense_gemm": None if dense_ms is None else round(dense_ms / mm_ms, 3),
+            "iteration_ms_with_soft_threshold_and_mvue_compress": round(step_ms, 4), "rel_err_vs_dense_fp32": rel}
+        torch.cuda.empty_cache()
+        sparse_ms, dense_step_ms, sl, dl, tf, one_pass_ms = train_workload(a.steps, a.warmup)
+        line["train_config4"] = {
+            "workload": "BASELINE configs[3]: SparseLinearTranspose GPT-2-124M MLP step, 12288 tokens, 768->3072->768, fp16 autocast, "
+                        "masked decay 2e-4, fused AdamW, mask refresh every 40 steps",
+            "ms_per_step": round(sparse_ms, 4), "ms_per_step_with_MaskedDecayAdamW": round(one_pass_ms, 4),
+            "dense_autocast_ms_per_step": round(dense_step_ms, 4), "speedup_vs_dense_step": round(dense_step_ms / sparse_ms, 3),
+            "speedup_vs_dense_step_with_MaskedDecayAdamW": round(dense_step_ms / one_pass_ms, 3),
+            "tflops_dense_equivalent": round(tf / (sparse_ms * 1e-3) / 1e12, 1), "final_loss": {"sparse": sl, "dense": dl}}
+        torch.cuda.empty_cache()
     if not a.no_convert:
         line["conversion_kernels_GBps"] = conversion_kernels()
     if not a.no_cpu:
-        line["cpu_baseline"] = cpu_baseline_spmm(min(os.cpu_count() or 1, 16))
+        line["cpu_baseline"] = cpu_baseline_spmm(host_threads())
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))
