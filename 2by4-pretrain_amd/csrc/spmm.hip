@@ -226,6 +226,9 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 // Workgroup ids are remapped so that the 8 XCDs (ids are dealt round-robin) each walk a
 // contiguous range of tiles in an 8-tile-high grouped raster: the ~32 tiles resident on an XCD
 // form an 8 x 4 patch that shares A rows and B columns in that XCD's L2.
+// With more tiles than compute units (and no k pieces) one workgroup per compute unit walks its
+// tiles in one pipeline (PERSIST): the copies of the next tile's first two stages ride in the last
+// two stages of the current one, and the output pass stages through the one buffer that is free.
 // At sustained clocks this kernel runs against the board's power limit (the shader clock settles
 // well below its 2.4 GHz maximum, the lower the more the operand bits toggle): what buys time is
 // fewer bytes moved per instruction, not a tighter schedule.
@@ -315,7 +318,12 @@ __device__ __forceinline__ void wait_copies_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <typename T, typename OutT, bool C_JMAJOR, typename C, bool B_KSTRIDED>
+// workgroup barrier behind this wave's LDS reads only: copies stay in flight
+__device__ __forceinline__ void wait_reads_and_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <typename T, typename OutT, bool C_JMAJOR, typename C, bool B_KSTRIDED, bool PERSIST>
 __global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
@@ -336,20 +344,30 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 
   // ---- XCD-aware work assignment.  A unit of work is (k-split, tile); units are ordered split-major
   // so that the units resident on an XCD belong to the same k range and share operand rows in L2.
+  // Workgroup ids are dealt to the 8 XCDs round-robin: XCD x owns the units [x * per_xcd, (x+1) * per_xcd),
+  // its workgroup number s = id / 8 takes unit s of that range -- and, PERSIST, every `slots`-th one after
+  // it (slots = workgroups per XCD), one tile after the other in the same pipeline.
   const int ntiles = tiles_i * tiles_j;
   const int nunits = ntiles * splits;
   const int per_xcd = (nunits + 7) / 8;
   const int bid = blockIdx.x;
-  const int unit = (bid & 7) * per_xcd + (bid >> 3);
-  if (unit >= nunits) return;
-  const int split = unit / ntiles, tile = unit - split * ntiles;
+  const int slots = PERSIST ? (int)(gridDim.x >> 3) : per_xcd;
+  const int xcd_end = min(((bid & 7) + 1) * per_xcd, nunits);
+  int unit = (bid & 7) * per_xcd + (bid >> 3);
+  if (unit >= xcd_end) return;
   constexpr int GH = C::GH;
-  const int group = tile / (GH * tiles_j);
-  const int gh = min(GH, tiles_i - group * GH);
-  const int in_group = tile - group * GH * tiles_j;
-  const int tile_i = group * GH + in_group % gh;
-  const int tile_j = in_group / gh;
-  const int64_t i0 = (int64_t)tile_i * C::BI, j0 = (int64_t)tile_j * C::BJ;
+  int split = 0;
+  int64_t i0 = 0, j0 = 0;
+  auto locate = [&](int u, int64_t& ti0, int64_t& tj0) {       // unit -> k piece and tile origin
+    split = u / ntiles;
+    const int tile = u - split * ntiles;
+    const int group = tile / (GH * tiles_j);
+    const int gh = min(GH, tiles_i - group * GH);
+    const int in_group = tile - group * GH * tiles_j;
+    ti0 = (int64_t)(group * GH + in_group % gh) * C::BI;
+    tj0 = (int64_t)(in_group / gh) * C::BJ;
+  };
+  locate(unit, i0, j0);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -365,40 +383,48 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   //    (and 256*M_ROW metadata bytes): copy q brings 16 rows x 64 bytes.
   const uint8_t* gb[C::NB];
   const uint8_t* ga[C::NA];
+  const uint8_t* gm[MW];
   // B with k strided (element (k,j) at k*ldb + j, 16-bit types): the stage is kept as [64 k][256 j]
   // in LDS, copy q brings 2 k-rows x 512 bytes; 16-byte chunks are XOR-swizzled with
   // ((k & 3) << 1) | ((k >> 3 & 1) << 3) so that the transposing fragment reads below (four k-rows x
   // 32 bytes per 16 lanes) touch every bank once.  Columns past n_dense re-read the last chunk.
   constexpr int64_t B_STAGE_ADVANCE_ROWS = B_KSTRIDED ? C::KB / ES : 0;
-#pragma unroll
-  for (int q = 0; q < C::NB; q++) {
-    if constexpr (B_KSTRIDED) {
-      const int krow = (wave * C::NB + q) * 2 + (lane >> 5);
-      const int ch = (lane & 31) ^ (((krow & 3) << 1) | (((krow >> 3) & 1) << 3));
-      const int64_t col = min(j0 + ch * 8, n_dense - 8);
-      gb[q] = b + ((int64_t)st_begin * B_STAGE_ADVANCE_ROWS + krow) * ldb_bytes + col * ES;
-    } else {
-      const int row = (wave * C::NB + q) * 8 + (lane >> 3);
-      const int ch = (lane & 7) ^ ((row >> 1) & 7);
-      gb[q] = b + min(j0 + row, n_dense - 1) * ldb_bytes + ch * 16 + (int64_t)st_begin * C::B_ROW;
-    }
-  }
   const int64_t b_stage_stride = B_KSTRIDED ? B_STAGE_ADVANCE_ROWS * ldb_bytes : (int64_t)C::B_ROW;
+  auto point_at = [&](int64_t ti0, int64_t tj0) {              // sources of the first stage of the tile at (ti0, tj0)
+    // (PERSIST: the lane id is made opaque here and in the output pass, so that the per-lane terms of the
+    // addresses are formed again for every tile instead of living in registers through the main loop,
+    // where the accumulators and two fragment sets leave none to spare)
+    int lane = threadIdx.x & 63;
+    if constexpr (PERSIST) asm volatile("" : "+v"(lane));
 #pragma unroll
-  for (int q = 0; q < C::NA; q++) {
-    const int row = (wave * C::NA + q) * 16 + (lane >> 2);
-    const int ch = (lane & 3) ^ ((row >> 2) & 3);
-    ga[q] = a_values + min(i0 + row, n_sparse - 1) * 64 + ch * 16 + (int64_t)st_begin * n_sparse * 64;
-  }
-  const uint8_t* gm[MW];
+    for (int q = 0; q < C::NB; q++) {
+      if constexpr (B_KSTRIDED) {
+        const int krow = (wave * C::NB + q) * 2 + (lane >> 5);
+        const int ch = (lane & 31) ^ (((krow & 3) << 1) | (((krow >> 3) & 1) << 3));
+        const int64_t col = min(tj0 + ch * 8, n_dense - 8);
+        gb[q] = b + ((int64_t)st_begin * B_STAGE_ADVANCE_ROWS + krow) * ldb_bytes + col * ES;
+      } else {
+        const int row = (wave * C::NB + q) * 8 + (lane >> 3);
+        const int ch = (lane & 7) ^ ((row >> 1) & 7);
+        gb[q] = b + min(tj0 + row, n_dense - 1) * ldb_bytes + ch * 16 + (int64_t)st_begin * C::B_ROW;
+      }
+    }
 #pragma unroll
-  for (int q = 0; q < MW; q++) {
-    const int d = (wave * MW + q) * 64 + lane;               // dword index in the stage's step-major metadata
-    constexpr int DW_PER_STEP = C::BI * M_STEP / 4;
-    const int step = d / DW_PER_STEP, r = d % DW_PER_STEP;
-    const int row = r / (M_STEP / 4), part = r % (M_STEP / 4);
-    gm[q] = a_meta + min(i0 + row, n_sparse - 1) * M_ROW + step * M_STEP + part * 4 + (int64_t)st_begin * n_sparse * M_ROW;
-  }
+    for (int q = 0; q < C::NA; q++) {
+      const int row = (wave * C::NA + q) * 16 + (lane >> 2);
+      const int ch = (lane & 3) ^ ((row >> 2) & 3);
+      ga[q] = a_values + min(ti0 + row, n_sparse - 1) * 64 + ch * 16 + (int64_t)st_begin * n_sparse * 64;
+    }
+#pragma unroll
+    for (int q = 0; q < MW; q++) {
+      const int d = (wave * MW + q) * 64 + lane;               // dword index in the stage's step-major metadata
+      constexpr int DW_PER_STEP = C::BI * M_STEP / 4;
+      const int step = d / DW_PER_STEP, r = d % DW_PER_STEP;
+      const int row = r / (M_STEP / 4), part = r % (M_STEP / 4);
+      gm[q] = a_meta + min(ti0 + row, n_sparse - 1) * M_ROW + step * M_STEP + part * 4 + (int64_t)st_begin * n_sparse * M_ROW;
+    }
+  };
+  point_at(i0, j0);
   const int64_t a_stage_stride = n_sparse * 64, m_stage_stride = n_sparse * M_ROW;
   constexpr int NCOPY = C::NB + C::NA + MW;      // copies per wave per stage
 
@@ -536,9 +562,22 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 
   issue(0, smem_at);
   if (nstages > 1) issue(1, smem_at + STAGE_BYTES);
+  uint32_t cur = 0, nxt = STAGE_BYTES, fre = 2 * STAGE_BYTES;   // buffers of stage st, st+1, st+2 (= st-1)
+  // PERSIST (nstages >= 4, no k pieces): the workgroup walks its tiles in one pipeline.  The copies of
+  // the next tile's first two stages are issued during the last two stages of the current one, into
+  // the two buffers those stages leave free; the output pass then stages through the third (the last
+  // stage's) while they fly, and the next tile starts with its operands already in LDS.
+  int next_unit = unit;
+  int64_t next_i0 = 0, next_j0 = 0;
+  bool has_next = false;
+  for (;;) {
+  // Also behind an output pass this wait is enough.  The counter of outstanding memory operations does
+  // not tell the pass's stores from copies, and stores may complete out of order with loads; but loads
+  // complete in order, and after the copies of stage s a wave issues the NCOPY copies of stage s + 1
+  // before it waits: if one copy of stage s were still in flight, all of those would be too, more
+  // than the NCOPY operations the wait allows.
   stage_barrier(nstages > 1);
   // stage 0: nothing to multiply yet
-  uint32_t cur = 0, nxt = STAGE_BYTES, fre = 2 * STAGE_BYTES;   // buffers of stage st, st+1, st+2 (= st-1)
   {
     const bool more = 2 < nstages;
 #pragma unroll
@@ -558,11 +597,24 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     mma_step(0, 1, true, st + 2, smem_at + fre, true, cur, 1);
     stage_barrier(true);
   }
-  for (; st < nstages; st++) {                    // the last two stages: nothing left to copy
+  if constexpr (PERSIST) {
+    next_unit = unit + slots;
+    has_next = next_unit < xcd_end;
+    if (has_next) {                                 // every copy of this tile has been issued: aim at the next one
+      locate(next_unit, next_i0, next_j0);
+      point_at(next_i0, next_j0);
+    }
+  }
+  for (; st < nstages; st++) {                    // the last two stages: nothing left to copy for this tile
     const uint32_t t = cur; cur = nxt; nxt = fre; fre = t;
-    mma_step(1, 0, false, 0, 0, true, cur, 0);
-    mma_step(0, 1, false, 0, 0, true, cur, 1);
-    stage_barrier(false);
+    const int pst = st - (nstages - 2);           // stage 0, then 1 of the next tile
+    mma_step(1, 0, has_next, pst, smem_at + fre, true, cur, 0);
+    mma_step(0, 1, has_next, pst, smem_at + fre, true, cur, 1);
+    // behind the last barrier of a tile no wave reads the stage buffers any more; the next tile's
+    // copies are not waited for here
+    if (st + 1 < nstages) stage_barrier(has_next);
+    else if (has_next) wait_reads_and_barrier();
+    else stage_barrier(false);
   }
   mma_step(1, 0, false, 0, 0, false, 0, 0);       // the last step
 
@@ -587,26 +639,29 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 
   auto output_pass = [&](auto mode_c) {
     constexpr int MODE = decltype(mode_c)::value;
+    int lane = threadIdx.x & 63;
+    if constexpr (PERSIST) asm volatile("" : "+v"(lane));
+    const int l32 = lane & 31, lh = lane >> 5;
     // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
     // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
     // (8 bytes) in 32 different output rows, so direct stores would touch 32 lines per instruction.
-    // Instead every wave stages 64(j) x 128(i) pieces of its sub-tile in a private 16 KB slice of the
-    // now idle B stage buffers (256-byte rows, 16-byte chunks XOR-swizzled with the row) and streams
-    // them out as four full 256-byte row segments per instruction (streaming stores: the tile is not
-    // read again by this kernel and should not displace operand lines in L2).
+    // Instead every wave stages 32(j) x 64(i) pieces of its sub-tile in a private 4 KB slice of the
+    // last stage's buffer (no wave reads it any more: the tile's last barrier is behind us; the other
+    // two buffers may already be receiving the next tile) -- 128-byte rows, 16-byte chunks
+    // XOR-swizzled with the row -- and streams them out as eight full 128-byte row segments per
+    // instruction (streaming stores: the tile is not read again by this kernel and should not
+    // displace operand lines in L2).  LDS accesses of one wave execute in order, so the passes need
+    // no barrier between them.
     if constexpr (C_JMAJOR && sizeof(OutT) == 2) {
-      __syncthreads();                                          // every wave is done with the stage buffers
-      uint8_t* stage = smem + wave * 16384;
-      const int rr = lane >> 4, chr = lane & 15;
-      const int64_t icol = i0 + wi * C::WI + chr * 8;
+      uint8_t* stage = smem + cur + wave * 4096;
+      const int rr = lane >> 3, chr = lane & 7;
   #pragma unroll
-      for (int half = 0; half < C::TJ / 2; half++) {            // 64 output rows (j) per pass
+      for (int tj = 0; tj < C::TJ; tj++) {
   #pragma unroll
-        for (int ti = 0; ti < C::TI; ti++)
+        for (int ip = 0; ip < C::TI / 2; ip++) {                // 64 sparse rows (i) per pass
   #pragma unroll
           for (int t2 = 0; t2 < 2; t2++) {
-            const int tj = half * 2 + t2;
-            const int jl = t2 * 32 + l32;
+            const int ti = ip * 2 + t2;
   #pragma unroll
             for (int g = 0; g < 4; g++) {
               const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
@@ -615,29 +670,30 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
               for (int r = 0; r < 4; r++) {
                 o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
               }
-              const int ch = ti * 4 + g;
-              *reinterpret_cast<Pack<OutT, 4>*>(stage + jl * 256 + ((ch ^ (jl & 15)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
+              const int ch = t2 * 4 + g;
+              *reinterpret_cast<Pack<OutT, 4>*>(stage + l32 * 128 + ((ch ^ (l32 & 7)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
             }
           }
+          const int64_t icol = i0 + wi * C::WI + ip * 64 + chr * 8;
   #pragma unroll
-        for (int it = 0; it < 16; it++) {
-          const int jl = it * 4 + rr;
-          const int64_t jrow = j0 + wj * C::WJ + half * 64 + jl;
-          const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 256 + ((chr ^ (jl & 15)) * 16));
-          if (jrow < n_dense && icol < n_sparse) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + jrow * ldc + icol));
+          for (int it = 0; it < 4; it++) {
+            const int jl = it * 8 + rr;
+            const int64_t jrow = j0 + wj * C::WJ + tj * 32 + jl;
+            const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 128 + ((chr ^ (jl & 7)) * 16));
+            if (jrow < n_dense && icol < n_sparse) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + jrow * ldc + icol));
+          }
         }
       }
     } else if constexpr (!C_JMAJOR && sizeof(OutT) == 2) {
       // i-major 16-bit output (the W.B of `S @ dense`): a lane owns single elements of 64+ different
-      // rows.  Stage 128(i) x 64(j) pieces as [i][64 j] (128-byte rows, chunks XOR-swizzled with the
+      // rows.  Stage 32(i) x 64(j) pieces as [i][64 j] (128-byte rows, chunks XOR-swizzled with the
       // row) and stream them out as eight full 128-byte rows per instruction.
-      __syncthreads();
-      uint8_t* stage = smem + wave * 16384;
+      uint8_t* stage = smem + cur + wave * 4096;
       const int rr = lane >> 3, chr = lane & 7;
   #pragma unroll
       for (int half = 0; half < C::TJ / 2; half++) {            // 64 output columns (j) per pass
   #pragma unroll
-        for (int ti = 0; ti < C::TI; ti++)
+        for (int ti = 0; ti < C::TI; ti++) {                    // 32 sparse rows (i) per pass
   #pragma unroll
           for (int t2 = 0; t2 < 2; t2++) {
             const int tj = half * 2 + t2;
@@ -646,19 +702,20 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             for (int g = 0; g < 4; g++)
   #pragma unroll
               for (int r = 0; r < 4; r++) {
-                const int il = ti * 32 + g * 8 + lh * 4 + r;
-                const int64_t row = i0 + wi * C::WI + il;
-                *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ ((il >> 1) & 7)) * 16) + (jl & 7) * 2) =
+                const int il = g * 8 + lh * 4 + r;
+                const int64_t row = i0 + wi * C::WI + ti * 32 + il;
+                *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ (il & 7)) * 16) + (jl & 7) * 2) =
                     to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row, row < n_sparse, act));
               }
           }
-        const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
+          const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
   #pragma unroll
-        for (int it = 0; it < 16; it++) {
-          const int il = it * 8 + rr;
-          const int64_t irow = i0 + wi * C::WI + il;
-          const int4v v = *reinterpret_cast<const int4v*>(stage + il * 128 + ((chr ^ ((il >> 1) & 7)) * 16));
-          if (irow < n_sparse && jcol < n_dense) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + irow * ldc + jcol));
+          for (int it = 0; it < 4; it++) {
+            const int il = it * 8 + rr;
+            const int64_t irow = i0 + wi * C::WI + ti * 32 + il;
+            const int4v v = *reinterpret_cast<const int4v*>(stage + il * 128 + ((chr ^ (il & 7)) * 16));
+            if (irow < n_sparse && jcol < n_dense) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + irow * ldc + jcol));
+          }
         }
       }
     } else {
@@ -689,6 +746,17 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   if (!bias && act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_PLAIN>{});
   else if (act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_BIAS>{});
   else output_pass(std::integral_constant<int, EPI_RUNTIME>{});
+  if (!has_next) break;
+  // ---- the next tile: its first two stages are (about to be) in the buffers nxt and fre
+  unit = next_unit; i0 = next_i0; j0 = next_j0;
+  { const uint32_t t = cur; cur = nxt; nxt = fre; fre = t; }
+#pragma unroll
+  for (int ti = 0; ti < C::TI; ti++)
+#pragma unroll
+    for (int tj = 0; tj < C::TJ; tj++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[ti][tj][r] = 0;
+  }
 }
 
 // Second pass of a split-K product: a block handles one eighth of a tile (the accumulator groups
@@ -773,6 +841,19 @@ TileCost tile_cost(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspa
   return {blocks, us};
 }
 
+// compute units of the current device (looked up once per device)
+inline int compute_units() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 template <typename T, typename OutT, typename C>
 int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
@@ -780,10 +861,23 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   const int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI), tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
   const int splits = workspace ? choose_splits<T, C>(n_sparse, k, n_dense, workspace_bytes) : 1;
   const int per_xcd = (tiles_i * tiles_j * splits + 7) / 8;
-  dim3 grid((unsigned)(per_xcd * 8));
+  // More tiles than compute units and no k pieces: one workgroup per compute unit walks its tiles in
+  // one pipeline (the next tile's operands arrive while the current one is written out).
+  const int cu_slots = compute_units() / 8;
+  const bool persist = C::BJ == 256 && sizeof(OutT) == 2 && c_layout == TF24_COL_MAJOR && splits == 1 &&
+                       k * (int64_t)sizeof(T) / C::KB >= 4 && per_xcd > cu_slots && cu_slots > 0;
+  dim3 grid((unsigned)((persist ? cu_slots : per_xcd) * 8));
   const bool jm = c_layout == TF24_COL_MAJOR;
   auto launch = [&](auto c_jmajor, auto b_kstrided) {
-    hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value>), grid, dim3(C::THREADS), 0, s,
+    if constexpr (C::BJ == 256 && sizeof(OutT) == 2 && decltype(c_jmajor)::value) {
+      if (persist) {
+        hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, true>), grid, dim3(C::THREADS), 0, s,
+                           (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                           (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
+        return;
+      }
+    }
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, false>), grid, dim3(C::THREADS), 0, s,
                        (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                        (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
   };

@@ -584,6 +584,31 @@ def test_dispatch_rules(cuda):
         s + 1
 
 
+@pytest.mark.parametrize("dtype,k", [(F16, 256), (F16, 320), (BF16, 704), (E4M3, 512), (E4M3, 640)])
+def test_spmm_chained_tiles_with_partial_edges(cuda, dtype, k):
+    """More 256 x 256 tiles than compute units: one workgroup per compute unit chains its tiles (the next
+    tile's first copies ride in the current tile's last two stages).  17 x 17 tiles with partial last
+    row and column of tiles, from the shortest k the chained form takes (4 stages) up; exact on small
+    integers, with and without bias, against the float32 product; 16-bit and 8-bit operands."""
+    import sparse
+    n, m = 4128, 4112
+    odt = torch.bfloat16 if dtype in FLOAT8 else dtype
+    w = _small_ints((n, k), 71, -2, 3).to(dtype)
+    x = _small_ints((m, k), 72, -2, 3).to(dtype)
+    bias = _small_ints((n,), 73).to(odt)
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    xg = x.to(cuda)
+    out = sparse.sparse_semi_structured_linear(xg, s, out_dtype=odt)
+    assert out.shape == (m, n) and out.float().cpu().equal(ref.to(odt).float())
+    out = sparse.sparse_semi_structured_linear(xg, s, bias_opt=bias.to(cuda), out_dtype=odt)
+    assert out.float().cpu().equal((ref + bias.float()).to(odt).float())
+    # twice in a row on the same buffers: nothing left over from the first launch
+    again = sparse.sparse_semi_structured_linear(xg, s, bias_opt=bias.to(cuda), out_dtype=odt)
+    assert again.equal(out)
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16, E4M3, E5M2])
 def test_spmm_tiled_all_operand_positions(cuda, dtype):
     """Shapes large enough for the tiled kernel, with partial tiles: both operand positions, both
