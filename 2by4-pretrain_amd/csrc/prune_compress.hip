@@ -16,7 +16,10 @@ namespace tf24 {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
+// 8-element units per lane of the row-major kernel.  One input stream (magnitude) is fastest with four
+// units per lane (37 against 43 us at 8192 x 8192 with one); with a second stream beside it (mask,
+// uniforms) one unit per lane and four times the blocks is (MVUE24 82 against 85 us, mask 67 against 71).
+template <int MODE> constexpr int unroll_for() { return MODE == TF24_PRUNE_MAGNITUDE ? 4 : 1; }
 
 // Kept-mask bits of one group; in MVUE mode also the inclusion probabilities the two kept
 // values are divided by.
@@ -57,6 +60,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
                    const MaskT* __restrict__ mask, int64_t mask_ld,
                    RandSrc rs,
                    Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift) {
+  constexpr int kUnroll = unroll_for<MODE>();
   constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
   const int64_t upr = k >> 3;                             // 8-element units per row
   const int64_t total = m * upr;
@@ -128,6 +132,81 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     w |= __shfl_down(mbyte, 2) << 16;
     w |= __shfl_down(mbyte, 3) << 24;
     if (live && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ounit) = w;
+  }
+}
+
+// Magnitude mode on 16-bit floats (the weight conversions of the configs): same work assignment and
+// outputs as prune_compress_row, with the selection done on the bit patterns (magnitude_top2_16:
+// a third of the instructions of the float compares) and the four dense loads of a lane issued
+// before the first is used: with one load in flight per wave the kernel is bound by memory latency,
+// a wave alternating between waiting for its load and computing.  A unit that holds a NaN is handed
+// to the float compares, whose answer for NaN the integer order does not give.
+template <typename In, typename Out>
+__global__ void __launch_bounds__(kThreads)
+prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
+                         Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift) {
+  constexpr int kUnroll = unroll_for<TF24_PRUNE_MAGNITUDE>();
+  constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
+  constexpr uint32_t kInf = std::is_same<In, f16_t>::value ? 0x7c00u : 0x7f80u;
+  const int64_t upr = k >> 3;
+  const int64_t total = m * upr;
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  bool live[kUnroll];
+  int64_t ounit[kUnroll];
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 in[kUnroll];
+#pragma unroll
+  for (int it = 0; it < kUnroll; it++) {
+    const int64_t u = base + (int64_t)it * kThreads;
+    int64_t row = 0, col8 = u;
+    live[it] = u < total;
+    if (panel) {
+      const int rpi = kThreads >> lpr_shift;
+      row = (int64_t)blockIdx.y * (kUnroll * rpi) + it * rpi + (threadIdx.x >> lpr_shift);
+      col8 = ((int64_t)blockIdx.x << lpr_shift) + (threadIdx.x & ((1 << lpr_shift) - 1));
+      live[it] = col8 < upr;
+      ounit[it] = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
+    } else {
+      if (!contiguous) {
+        row = (int64_t)((uint32_t)u / (uint32_t)upr);
+        col8 = u - row * upr;
+      }
+      ounit[it] = row * upr + col8;
+    }
+    in[it] = u32x4{0, 0, 0, 0};
+    if (live[it]) in[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dense + row * ld + col8 * 8));
+  }
+#pragma unroll
+  for (int it = 0; it < kUnroll; it++) {
+    const uint32_t w0 = in[it][0], w1 = in[it][1], w2 = in[it][2], w3 = in[it][3];
+    const Top2 t0 = magnitude_top2_16(w0, w1), t1 = magnitude_top2_16(w2, w3);
+    uint32_t n0 = t0.nibble, n1 = t1.nibble;
+    if (max(t0.top_key, t1.top_key) > ((kInf << 2) | 3u)) {          // a NaN in the unit
+      const In* e = reinterpret_cast<const In*>(&in[it]);
+      n0 = encode_nibble(magnitude_mask4(to_float(e[0]), to_float(e[1]), to_float(e[2]), to_float(e[3])));
+      n1 = encode_nibble(magnitude_mask4(to_float(e[4]), to_float(e[5]), to_float(e[6]), to_float(e[7])));
+    }
+    const uint32_t r0 = pick16(w0, w1, n0 & 3u), r1 = pick16(w0, w1, n0 >> 2);
+    const uint32_t r2 = pick16(w2, w3, n1 & 3u), r3 = pick16(w2, w3, n1 >> 2);
+    Pack<Out, 4> out;
+    if constexpr (std::is_same<In, Out>::value) {
+      uint32_t* o = reinterpret_cast<uint32_t*>(out.v);
+      o[0] = (r0 & 0xffffu) | (r1 << 16);
+      o[1] = (r2 & 0xffffu) | (r3 << 16);
+    } else {
+      out.v[0] = from_float<Out>(to_float(In{(uint16_t)r0}));
+      out.v[1] = from_float<Out>(to_float(In{(uint16_t)r1}));
+      out.v[2] = from_float<Out>(to_float(In{(uint16_t)r2}));
+      out.v[3] = from_float<Out>(to_float(In{(uint16_t)r3}));
+    }
+    if (live[it]) out.store_stream(values + ounit[it] * 4);
+    // 4 adjacent lanes (32 dense columns of one row) -> one metadata dword
+    const uint32_t mbyte = live[it] ? n0 | (n1 << 4) : 0u;
+    uint32_t w = mbyte;
+    w |= __shfl_down(mbyte, 1) << 8;
+    w |= __shfl_down(mbyte, 2) << 16;
+    w |= __shfl_down(mbyte, 3) << 24;
+    if (live[it] && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ounit[it]) = w;
   }
 }
 
@@ -308,6 +387,7 @@ template <typename In, typename Out, int MODE, typename MaskT>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
            RandSrc rs, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t stream) {
   if (layout == TF24_ROW_MAJOR) {
+    constexpr int kUnroll = unroll_for<MODE>();
     const int64_t per_block = kThreads * kUnroll;
     const bool contiguous = ld == k && (MODE != TF24_PRUNE_MASK || mask_ld == k) && (MODE != TF24_PRUNE_MVUE || rs.kind == RAND_SEEDED || rs.ld == (rs.kind == RAND_PACKED ? k / 2 : k));
     const int64_t total = m * (k >> 3);
@@ -319,9 +399,14 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
       const int rows_per_block = kUnroll * (kThreads >> lpr_shift), units_per_block = 1 << lpr_shift;
       grid = dim3((unsigned)(((k >> 3) + units_per_block - 1) / units_per_block), (unsigned)(m / rows_per_block));
     }
-    hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
-                       (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rs, (Out*)values, (uint8_t*)meta,
-                       contiguous, panel, lpr_shift);
+    if constexpr (MODE == TF24_PRUNE_MAGNITUDE && (std::is_same<In, f16_t>::value || std::is_same<In, bf16_t>::value)) {
+      hipLaunchKernelGGL((prune_compress_row_mag16<In, Out>), grid, dim3(kThreads), 0, stream,
+                         (const In*)dense, ld, m, k, (Out*)values, (uint8_t*)meta, contiguous, panel, lpr_shift);
+    } else {
+      hipLaunchKernelGGL((prune_compress_row<In, Out, MODE, MaskT>), grid, dim3(kThreads), 0, stream,
+                         (const In*)dense, ld, m, k, (const MaskT*)mask, mask_ld, rs, (Out*)values, (uint8_t*)meta,
+                         contiguous, panel, lpr_shift);
+    }
   } else {
     constexpr int R = 16 / sizeof(In);
     dim3 grid((unsigned)((m + 8 * R - 1) / (8 * R)), (unsigned)((k + 127) / 128));

@@ -202,6 +202,32 @@ __device__ __forceinline__ uint32_t encode_nibble(uint32_t mbits) {
   return (uint32_t)bit0 | ((uint32_t)bit1 << 1) | ((uint32_t)bit2 << 2) | ((uint32_t)bit3 << 3);
 }
 
+// Magnitude selection of one group of four 16-bit floats (f16 or bf16) held as two dwords
+// (x1:x0, x3:x2), in integer arithmetic: for numbers the order of |x| is the order of the low 15
+// bits, so key_i = |bits_i| << 2 | i orders the elements by (|x|, index) -- exactly the rule of the
+// six compares (a tie keeps the larger index) -- and the two kept elements are the largest and the
+// second largest key: four min/max pairs, a max and a max3.  Returns the nibble pos0 | pos1 << 2;
+// `top_key` (largest key) lets the caller test for NaN, whose magnitude bits lie above infinity's:
+// a group with a NaN follows the float compares instead (NaN compares false either way there).
+// About 20 instructions against about 60 for compares, lane-mask logic and the table encoding.
+struct Top2 { uint32_t nibble, top_key; };
+__device__ __forceinline__ Top2 magnitude_top2_16(uint32_t lo, uint32_t hi) {
+  const uint32_t k0 = (lo & 0x7fffu) << 2;
+  const uint32_t k1 = (((lo >> 16) & 0x7fffu) << 2) | 1u;
+  const uint32_t k2 = ((hi & 0x7fffu) << 2) | 2u;
+  const uint32_t k3 = (((hi >> 16) & 0x7fffu) << 2) | 3u;
+  const uint32_t hi01 = max(k0, k1), lo01 = min(k0, k1), hi23 = max(k2, k3), lo23 = min(k2, k3);
+  const uint32_t top = max(hi01, hi23);
+  const uint32_t second = max(min(hi01, hi23), max(lo01, lo23));
+  const uint32_t p = top & 3u, q = second & 3u;
+  return {min(p, q) | (max(p, q) << 2), top};
+}
+// the 16-bit element at position pos (0..3) of the group (x1:x0, x3:x2), in the low half of the result
+__device__ __forceinline__ uint32_t pick16(uint32_t lo, uint32_t hi, uint32_t pos) {
+  const uint64_t both = ((uint64_t)hi << 32) | lo;
+  return (uint32_t)(both >> (pos << 4));
+}
+
 template <typename T>
 __device__ __forceinline__ T select4(uint32_t pos, T v0, T v1, T v2, T v3) {
   T lo = (pos & 1) ? v1 : v0;
