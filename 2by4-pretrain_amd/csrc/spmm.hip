@@ -304,12 +304,15 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 __device__ __forceinline__ uint32_t lds_offset(const void* p) {
   return (uint32_t)(uintptr_t)(lds_ptr_t)p;
 }
-__device__ __forceinline__ void g2l16(const uint8_t* g, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
+// The source address is a wave-uniform 64-bit base in scalar registers plus a 32-bit offset per lane: with a
+// 64-bit address per lane the same copies hold up the matrix instructions issued around them (on an
+// instruction mix like the main loop's, 25 % more cycles than the matrix instructions alone against 3 %).
+__device__ __forceinline__ void g2l16(const uint8_t* base, uint32_t lane_offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
 }
 // same with one dword per lane: lane l writes LDS[base + 4*l]
-__device__ __forceinline__ void g2l4(const uint8_t* g, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_base) : "memory", "m0");
+__device__ __forceinline__ void g2l4(const uint8_t* base, uint32_t lane_offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
 }
 // s_waitcnt vmcnt(N) + s_barrier with a compile-time N (a bare s_barrier: __syncthreads() would add
 // a fence that drains every outstanding copy)
@@ -334,7 +337,11 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   constexpr int M_STEP = M_ROW / C::STEPS;
   // Metadata is copied one dword per lane (256 bytes per wave instruction) so that it can be laid
   // out step-major in LDS, [step][row][M_STEP bytes]: the index words the 32 rows of a wave read for
-  // one step are then consecutive and conflict-free (row-major, 8 bytes apart, two rows share a bank).
+  // one step are then consecutive and conflict-free.  16-bit values: [step][row][4 bytes], a lane reads the
+  // halfword of its k half.  8-bit values (a dword per lane and k half): [step][k half][row][4 bytes], so
+  // that the 32 lanes of a half read 128 consecutive bytes -- row-major 8-byte entries put rows r and
+  // r + 16 of a 32-lane pass on one bank and every index read took two passes more.
+  constexpr bool M_HALF_MAJOR = ES == 1;
   constexpr int MW = C::BI * M_ROW / 256 / C::NW;           // dword copies per wave per stage (1 or 2)
   static_assert(MW * 256 * C::NW == C::BI * M_ROW, "metadata copies must divide among the waves");
   // one stage buffer = [A values | B | A metadata]; three of them rotate
@@ -381,9 +388,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // B: copy q of a wave brings 8 rows x 128 bytes; lane -> (row, swizzled chunk).
   // A: stage st of rows i0..i0+255 is one contiguous run of 256*64 value bytes at (st*n_sparse + i0)*64
   //    (and 256*M_ROW metadata bytes): copy q brings 16 rows x 64 bytes.
-  const uint8_t* gb[C::NB];
-  const uint8_t* ga[C::NA];
-  const uint8_t* gm[MW];
+  // Every source is (tile base, uniform, advanced by whole stages) + (lane offset inside the tile's first stage).
+  uint32_t ob[C::NB], oa[C::NA], om[MW];
+  const uint8_t *tile_b, *tile_a, *tile_m;
   // B with k strided (element (k,j) at k*ldb + j, 16-bit types): the stage is kept as [64 k][256 j]
   // in LDS, copy q brings 2 k-rows x 512 bytes; 16-byte chunks are XOR-swizzled with
   // ((k & 3) << 1) | ((k >> 3 & 1) << 3) so that the transposing fragment reads below (four k-rows x
@@ -396,32 +403,37 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     // where the accumulators and two fragment sets leave none to spare)
     int lane = threadIdx.x & 63;
     if constexpr (PERSIST) asm volatile("" : "+v"(lane));
+    const int64_t last_j = n_dense - 1 - tj0, last_i = n_sparse - 1 - ti0;       // >= 0: tile origins lie inside
+    if constexpr (B_KSTRIDED) tile_b = b + (int64_t)st_begin * B_STAGE_ADVANCE_ROWS * ldb_bytes;   // columns stay absolute: the clamp may step left of the tile
+    else tile_b = b + tj0 * ldb_bytes + (int64_t)st_begin * C::B_ROW;
+    tile_a = a_values + (ti0 + (int64_t)st_begin * n_sparse) * 64;
+    tile_m = a_meta + (ti0 + (int64_t)st_begin * n_sparse) * M_ROW;
 #pragma unroll
     for (int q = 0; q < C::NB; q++) {
       if constexpr (B_KSTRIDED) {
         const int krow = (wave * C::NB + q) * 2 + (lane >> 5);
         const int ch = (lane & 31) ^ (((krow & 3) << 1) | (((krow >> 3) & 1) << 3));
         const int64_t col = min(tj0 + ch * 8, n_dense - 8);
-        gb[q] = b + ((int64_t)st_begin * B_STAGE_ADVANCE_ROWS + krow) * ldb_bytes + col * ES;
+        ob[q] = (uint32_t)(krow * ldb_bytes + col * ES);
       } else {
         const int row = (wave * C::NB + q) * 8 + (lane >> 3);
         const int ch = (lane & 7) ^ ((row >> 1) & 7);
-        gb[q] = b + min(tj0 + row, n_dense - 1) * ldb_bytes + ch * 16 + (int64_t)st_begin * C::B_ROW;
+        ob[q] = (uint32_t)(min((int64_t)row, last_j) * ldb_bytes + ch * 16);
       }
     }
 #pragma unroll
     for (int q = 0; q < C::NA; q++) {
       const int row = (wave * C::NA + q) * 16 + (lane >> 2);
       const int ch = (lane & 3) ^ ((row >> 2) & 3);
-      ga[q] = a_values + min(ti0 + row, n_sparse - 1) * 64 + ch * 16 + (int64_t)st_begin * n_sparse * 64;
+      oa[q] = (uint32_t)(min((int64_t)row, last_i) * 64 + ch * 16);
     }
 #pragma unroll
     for (int q = 0; q < MW; q++) {
       const int d = (wave * MW + q) * 64 + lane;               // dword index in the stage's step-major metadata
       constexpr int DW_PER_STEP = C::BI * M_STEP / 4;
       const int step = d / DW_PER_STEP, r = d % DW_PER_STEP;
-      const int row = r / (M_STEP / 4), part = r % (M_STEP / 4);
-      gm[q] = a_meta + min(ti0 + row, n_sparse - 1) * M_ROW + step * M_STEP + part * 4 + (int64_t)st_begin * n_sparse * M_ROW;
+      const int row = M_HALF_MAJOR ? r % C::BI : r / (M_STEP / 4), part = M_HALF_MAJOR ? r / C::BI : r % (M_STEP / 4);
+      om[q] = (uint32_t)(min((int64_t)row, last_i) * M_ROW + step * M_STEP + part * 4);
     }
   };
   point_at(i0, j0);
@@ -431,9 +443,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // copy q of this wave for stage st into the stage buffer at LDS byte address `dst`
   const uint32_t smem_at = lds_offset(smem);
   auto issue_one = [&](int q, int st, uint32_t dst) {
-    if (q < C::NB) g2l16(gb[q] + (int64_t)st * b_stage_stride, dst + B_AT + (wave * C::NB + q) * 1024);
-    else if (q < C::NB + C::NA) g2l16(ga[q - C::NB] + (int64_t)st * a_stage_stride, dst + (wave * C::NA + q - C::NB) * 1024);
-    else g2l4(gm[q - C::NB - C::NA] + (int64_t)st * m_stage_stride, dst + M_AT + (wave * MW + q - C::NB - C::NA) * 256);
+    if (q < C::NB) g2l16(tile_b + (int64_t)st * b_stage_stride, ob[q], dst + B_AT + (wave * C::NB + q) * 1024);
+    else if (q < C::NB + C::NA) g2l16(tile_a + (int64_t)st * a_stage_stride, oa[q - C::NB], dst + (wave * C::NA + q - C::NB) * 1024);
+    else g2l4(tile_m + (int64_t)st * m_stage_stride, om[q - C::NB - C::NA], dst + M_AT + (wave * MW + q - C::NB - C::NA) * 256);
   };
   auto issue = [&](int st, uint32_t dst) {
 #pragma unroll
@@ -458,7 +470,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
 #pragma unroll
     for (int h = 0; h < 2; h++) b_off[step][h] = b_row * C::B_ROW + (((step * 4 + h * 2 + lh) ^ b_sw) * 16);
   }
-  const int m_off = a_row * M_STEP + lh * (M_STEP / 2);          // inside a step's [row][M_STEP] block
+  const int m_off = M_HALF_MAJOR ? lh * (C::BI * 4) + a_row * 4 : a_row * M_STEP + lh * (M_STEP / 2);   // inside a step's block
+  constexpr int M_FRAG = M_HALF_MAJOR ? 32 * 4 : 32 * M_STEP;    // from one 32-row fragment to the next
   // k-strided B: transposing reads (DS_READ_B64_TR_B16).  In a group of 16 lanes, lane i receives
   // the halfwords i%4 of the source lanes 4e + i/4 (e = 0..3).  Source lane s therefore addresses
   // k-row k0 + s/4, halfwords 4*(s%4).. of the group's 16 columns, and lane i ends up with
@@ -514,8 +527,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     } else {
       const int f = (n - B_READS) >> 1;
       if (((n - B_READS) & 1) == 0) af[set][f] = *reinterpret_cast<const int4v*>(base + a_off[step] + f * 32 * C::A_ROW);
-      else if constexpr (ES == 2) idx[set][f] = *reinterpret_cast<const uint16_t*>(base + M_AT + m_off + f * 32 * M_STEP + step * (C::BI * M_STEP));
-      else idx[set][f] = *reinterpret_cast<const int*>(base + M_AT + m_off + f * 32 * M_STEP + step * (C::BI * M_STEP));
+      else if constexpr (ES == 2) idx[set][f] = *reinterpret_cast<const uint16_t*>(base + M_AT + m_off + f * M_FRAG + step * (C::BI * M_STEP));
+      else idx[set][f] = *reinterpret_cast<const int*>(base + M_AT + m_off + f * M_FRAG + step * (C::BI * M_STEP));
     }
   };
   // `half` selects which half of the wave's copies of stage pst is issued between the instructions
@@ -1252,6 +1265,8 @@ extern "C" int tf24_spmm_validate(int dtype, int64_t n_sparse, int64_t k, int b_
   if (c_layout != TF24_ROW_MAJOR && c_layout != TF24_COL_MAJOR) return fail(TF24_ERR_ARG, "%s: bad c_layout %d", fn, c_layout);
   const int64_t bext = b_layout == TF24_ROW_MAJOR ? k : n_dense;
   if (ldb < bext || ldb % dmult) return fail(TF24_ERR_STRIDE, "%s: ldb %lld must be >= %lld and a multiple of %lld", fn, (long long)ldb, (long long)bext, (long long)dmult);
+  // the copies address a tile's rows of B by 32-bit lane offsets from the tile's base: 256 rows must span < 4 GiB
+  if (ldb * (eight ? 1 : 2) > ((int64_t)1 << 24)) return fail(TF24_ERR_STRIDE, "%s: ldb %lld exceeds 16 MiB per row", fn, (long long)ldb);
   const int64_t cext = c_layout == TF24_ROW_MAJOR ? n_dense : n_sparse;
   // rows of the output leave as 16-byte stores: 8 elements of a 16-bit type, 4 of a 32-bit one
   const int64_t cmult = (out_dtype == TF24_F16 || out_dtype == TF24_BF16) ? 8 : 4;
