@@ -94,6 +94,8 @@ def test_transposable_and_spmm_validators(native):
     assert sp(N.F16, 32, 64, 8, ldb=32) == -3 and sp(N.F16, 32, 64, 8, ldc=16) == -3
     # output rows leave as 16-byte segments: ldc % 8 for 16-bit results, % 4 for 32-bit ones
     assert sp(N.F16, 32, 64, 8, ldc=36) == -3 and sp(N.F16, 32, 64, 8, ldc=40) == 0 and sp(N.F16, 32, 64, 8, ldc=36, out=N.F32) == 0
+    assert sp(N.F16, 32, 64, 8, ldb=1 << 23) == 0 and sp(N.F16, 32, 64, 8, ldb=(1 << 23) + 8) == -3     # rows of the dense operand: at most 16 MiB
+    assert sp(N.E4M3, 32, 128, 16, ldb=1 << 24) == 0 and sp(N.E4M3, 32, 128, 16, ldb=(1 << 24) + 16) == -3
     assert sp(N.F16, 32, 64, 8, act=5) == -5 and sp(N.F16, 32, 64, 8, bl=3) == -5
 
 
