@@ -568,6 +568,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     }
   };
   static_assert(C::STEPS == 2, "the pipeline below is written for two instruction steps per stage");
+  static_assert(!PERSIST || (C_JMAJOR && sizeof(OutT) == 2), "chained tiles rely on the wait inside the j-major 16-bit output pass");
   auto stage_barrier = [&](bool more) {          // B(st+1): only this wave's copies of stage st+2 may still fly
     if (!more) wait_copies_and_barrier<0>();
     else wait_copies_and_barrier<NCOPY>();
@@ -583,13 +584,17 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   int next_unit = unit;
   int64_t next_i0 = 0, next_j0 = 0;
   bool has_next = false;
+  bool chained = false;                          // this tile's first two stages were copied under the previous tile
   for (;;) {
-  // Also behind an output pass this wait is enough.  The counter of outstanding memory operations does
-  // not tell the pass's stores from copies, and stores may complete out of order with loads; but loads
-  // complete in order, and after the copies of stage s a wave issues the NCOPY copies of stage s + 1
-  // before it waits: if one copy of stage s were still in flight, all of those would be too, more
-  // than the NCOPY operations the wait allows.
-  stage_barrier(nstages > 1);
+  // A chained tile's first two stages were waited for by every wave before the first store of the previous
+  // output pass (below), so its first two barriers only publish them: waiting here on the counter of
+  // outstanding memory operations would wait for the acknowledgements of those stores, which it does not
+  // tell from copies.  From the third barrier on the usual wait is enough again: stores may complete out of
+  // order with loads, but loads complete in order, and after the copies of stage s a wave issues the NCOPY
+  // copies of stage s + 1 before it waits -- if one copy of stage s were still in flight, all of those
+  // would be too, more than the NCOPY operations the wait allows.
+  if (PERSIST && chained) wait_reads_and_barrier();
+  else stage_barrier(nstages > 1);
   // stage 0: nothing to multiply yet
   {
     const bool more = 2 < nstages;
@@ -600,7 +605,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
       for (int q = 0; q < C::TI * PER_SLOT && q < NCOPY; q++) issue_one(q, 2, smem_at + fre);
     }
     mma_step(0, 1, more, 2, smem_at + fre, true, cur, 1);
-    stage_barrier(more);
+    if (PERSIST && chained) wait_reads_and_barrier();
+    else stage_barrier(more);
   }
   // stage st: behind B(st), register set 1 holds the last step of stage st-1
   int st = 1;
@@ -688,6 +694,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             }
           }
           const int64_t icol = i0 + wi * C::WI + ip * 64 + chr * 8;
+          // the next tile's first two stages (issued one and two stages ago) have to be in LDS before this
+          // wave's first store joins the outstanding operations
+          if (PERSIST && tj == 0 && ip == 0 && has_next) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   #pragma unroll
           for (int it = 0; it < 4; it++) {
             const int jl = it * 8 + rr;
@@ -761,7 +770,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   else output_pass(std::integral_constant<int, EPI_RUNTIME>{});
   if (!has_next) break;
   // ---- the next tile: its first two stages are (about to be) in the buffers nxt and fre
-  unit = next_unit; i0 = next_i0; j0 = next_j0;
+  unit = next_unit; i0 = next_i0; j0 = next_j0; chained = true;
   { const uint32_t t = cur; cur = nxt; nxt = fre; fre = t; }
 #pragma unroll
   for (int ti = 0; ti < C::TI; ti++)

@@ -58,11 +58,11 @@ template <> __device__ __forceinline__ float from_float<float>(float f) { return
 template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) {
   return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};
 }
+// gfx950's V_CVT_PK_BF16_F32: round to nearest even, NaNs quieted with their upper payload bits kept --
+// on all 2^32 float32 patterns the same bits as the integer sequence (u + 0x7fff + (u >> 16 & 1)) >> 16 with
+// (u >> 16) | 0x40 for NaNs, in one instruction per pair instead of seven per value.
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)((u >> 16) | 0x40)};  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return bf16_t{(uint16_t)(u >> 16)};
+  return bf16_t{__builtin_bit_cast(uint16_t, (__bf16)f)};
 }
 // OCP e4m3fn (bias 7, no inf, 0x7f = NaN, max 448): values that round past 448 become NaN,
 // exactly like the bit pattern arithmetic of a round-to-nearest-even narrowing.
