@@ -15,8 +15,8 @@ template <typename T, bool PANEL>
 __global__ void __launch_bounds__(kThreads)
 decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta, int64_t total_units, int64_t m, int64_t k,
                   uint32_t chunks, T* __restrict__ dense) {
-  int64_t u, src;
-  if constexpr (PANEL) {        // [k/KP][m][KP/8 units]
+  int64_t u, src, msrc;          // dense unit, its place among the values, byte offset of its metadata byte
+  if constexpr (PANEL) {        // values [k/KP][m][KP/8 units], metadata [k/32][m][4 bytes]
     constexpr int UPP = (128 / (int)sizeof(T)) / 8;
     const int64_t upr = k >> 3;
     const uint32_t by = blockIdx.x / chunks, bx = blockIdx.x - by * chunks;        // chunks = 32-unit pieces of a row
@@ -24,14 +24,16 @@ decompress_kernel(const T* __restrict__ values, const uint8_t* __restrict__ meta
     if (col8 >= upr || row >= m) return;
     u = row * upr + col8;
     src = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
+    msrc = panel_meta_offset(col8, row, m);
   } else {
     u = (int64_t)blockIdx.x * kThreads + threadIdx.x;   // unit = 8 dense elements, row-major order
     if (u >= total_units) return;
     src = u;
+    msrc = u;
   }
   Pack<T, 4> v;
   v.load_stream(values + src * 4);
-  const uint32_t mb = meta[src];
+  const uint32_t mb = meta[msrc];
   Pack<T, 8> out;
 #pragma unroll
   for (int i = 0; i < 8; i++) out.v[i] = T{};
@@ -63,8 +65,9 @@ int launch(const void* values, const void* meta, bool panel, int64_t m, int64_t 
   return check_launch("tf24_decompress");
 }
 
-// Canonical <-> panel storage of a compressed operand.  Per row and panel the 64 value bytes and the
-// KP/8 metadata bytes are the same in both forms, only their place differs.  A block moves 8 rows x
+// Canonical <-> panel storage of a compressed operand.  Per row and panel the 64 value bytes are the
+// same in both forms, only their place differs; the metadata moves as 4-byte words (canonical: the row's
+// words in a row; panel: [k/32][m]).  A block moves 8 rows x
 // 8 panels: a wave the values of 2 rows x 8 panels, 16 bytes per lane (canonical side: 512
 // contiguous bytes per row; panel side: the two rows' adjacent pieces, one cache line per panel);
 // the first wave also the 64 metadata pieces, lane = (row, panel) (64- or 128-byte runs on both sides).
@@ -86,10 +89,12 @@ repack_kernel(const uint8_t* __restrict__ vin, const uint8_t* __restrict__ min_,
   if (wave == 0) {
     const int64_t p = (int64_t)bx * 8 + (lane & 7), row = (int64_t)by * 8 + (lane >> 3);
     if (p < panels && row < m) {
-      const int64_t canon = row * panels + p, panel = p * m + row;
-      const int64_t src = to_panel ? canon : panel, dst = to_panel ? panel : canon;
-      using Piece = typename std::conditional<META_BYTES == 16, uint4, uint2>::type;
-      *reinterpret_cast<Piece*>(mout + dst * META_BYTES) = *reinterpret_cast<const Piece*>(min_ + src * META_BYTES);
+#pragma unroll
+      for (int w = 0; w < META_BYTES / 4; w++) {
+        const int64_t canon = (row * panels + p) * META_BYTES + 4 * w, panel = ((p * (META_BYTES / 4) + w) * m + row) * 4;
+        const int64_t src = to_panel ? canon : panel, dst = to_panel ? panel : canon;
+        *reinterpret_cast<uint32_t*>(mout + dst) = *reinterpret_cast<const uint32_t*>(min_ + src);
+      }
     }
   }
 }
@@ -107,8 +112,8 @@ extern "C" int tf24_repack(const void* values_in, const void* meta_in, int dtype
   if (from_layout != TF24_COMPRESSED_CANONICAL && from_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, from_layout);
   if (!values_in || !meta_in || !values_out || !meta_out) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
   if (values_in == values_out || meta_in == meta_out) return fail(TF24_ERR_ARG, "%s: in-place conversion is not supported", fn);
-  if (((uintptr_t)values_in | (uintptr_t)values_out) % 16 || ((uintptr_t)meta_in | (uintptr_t)meta_out) % (kp / 8))
-    return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte and metadata %lld-byte aligned", fn, (long long)(kp / 8));
+  if (((uintptr_t)values_in | (uintptr_t)values_out) % 16 || ((uintptr_t)meta_in | (uintptr_t)meta_out) % 4)
+    return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte and metadata 4-byte aligned", fn);
   const int64_t panels = k / kp, chunks = (panels + 7) / 8, blocks = chunks * ((m + 7) / 8);
   if (blocks > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "%s: matrix too large", fn);
   const bool to_panel = from_layout == TF24_COMPRESSED_CANONICAL;

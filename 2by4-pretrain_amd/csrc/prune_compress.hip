@@ -49,8 +49,8 @@ __device__ __forceinline__ float kept_value(uint32_t pos, const float (&x)[4], c
 // ------------------------------------------------------------------ row-major
 // panel = false: canonical output, values [m, k/2] and metadata [m, k/8 bytes] row-major; units
 //   (8 dense elements) are walked along rows.
-// panel = true : panel output, [k/KP][m][64 bytes] values and [k/KP][m][KP/8 bytes] metadata with
-//   KP = 128 / sizeof(Out) dense elements per panel.  A block covers 64 rows x 128 dense columns
+// panel = true : panel output, [k/KP][m][64 bytes] values (KP = 128 / sizeof(Out) dense elements per
+//   panel) and [k/32][m][4 bytes] metadata.  A block covers 64 rows x 128 dense columns
 //   (32 x 256 when m is not a multiple of 64): 2^lpr_shift lanes read consecutive columns of one row,
 //   the other lanes of the wave take the next rows, so that every store instruction writes, per
 //   panel, the contiguous 64-byte pieces of 4 (2) adjacent rows.
@@ -71,7 +71,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     bool live = u < total;
     uint32_t mbyte = 0;
     Pack<Out, 4> out;
-    int64_t row = 0, col8 = 0, ounit = 0;
+    int64_t row = 0, col8 = 0, ounit = 0, ometa = 0;       // unit index among the values, byte offset of its metadata byte
     if (panel) {
       const int rpi = kThreads >> lpr_shift;                 // rows per iteration
       // blocks that run together (consecutive blockIdx.x) read neighbouring column ranges of the same rows
@@ -82,6 +82,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     if (live) {
       if (panel) {
         ounit = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
+        ometa = panel_meta_offset(col8, row, m);
       } else {
         if (contiguous) {          // every leading dimension equals k: offsets are linear in u
           col8 = u;
@@ -90,6 +91,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
           col8 = u - row * upr;
         }
         ounit = row * upr + col8;
+        ometa = ounit;
       }
       Pack<In, 8> in;
       in.load_stream(dense + row * ld + col8 * 8);
@@ -131,7 +133,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     w |= __shfl_down(mbyte, 1) << 8;
     w |= __shfl_down(mbyte, 2) << 16;
     w |= __shfl_down(mbyte, 3) << 24;
-    if (live && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ounit) = w;
+    if (live && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ometa) = w;
   }
 }
 
@@ -152,7 +154,7 @@ prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, in
   const int64_t total = m * upr;
   const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
   bool live[kUnroll];
-  int64_t ounit[kUnroll];
+  int64_t ounit[kUnroll], ometa[kUnroll];
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   u32x4 in[kUnroll];
 #pragma unroll
@@ -166,12 +168,14 @@ prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, in
       col8 = ((int64_t)blockIdx.x << lpr_shift) + (threadIdx.x & ((1 << lpr_shift) - 1));
       live[it] = col8 < upr;
       ounit[it] = ((col8 / UPP) * m + row) * UPP + col8 % UPP;
+      ometa[it] = panel_meta_offset(col8, row, m);
     } else {
       if (!contiguous) {
         row = (int64_t)((uint32_t)u / (uint32_t)upr);
         col8 = u - row * upr;
       }
       ounit[it] = row * upr + col8;
+      ometa[it] = ounit[it];
     }
     in[it] = u32x4{0, 0, 0, 0};
     if (live[it]) in[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dense + row * ld + col8 * 8));
@@ -206,7 +210,7 @@ prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, in
     w |= __shfl_down(mbyte, 1) << 8;
     w |= __shfl_down(mbyte, 2) << 16;
     w |= __shfl_down(mbyte, 3) << 24;
-    if (live[it] && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ounit[it]) = w;
+    if (live[it] && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ometa[it]) = w;
   }
 }
 
@@ -318,7 +322,6 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
   constexpr int LANES_PER_ROW = VROW_BYTES / 16;
   constexpr int ROWS_PER_PASS = kThreads / LANES_PER_ROW;
   constexpr int KP = 128 / (int)sizeof(Out);
-  constexpr int MP = KP / 8;                             // metadata bytes per row per panel
   const int64_t vpitch_out = (k >> 1) * sizeof(Out);
 #pragma unroll
   for (int pass = 0; pass < (TR + ROWS_PER_PASS - 1) / ROWS_PER_PASS; pass++) {
@@ -349,13 +352,9 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
         if (full) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(sp[2], sp[3]);
       } else {
         const int64_t mbyte0 = col0 >> 3;                // byte offset inside the row's canonical stream
-        uint8_t* dst = meta + ((mbyte0 / MP) * m + gr) * MP + (mbyte0 % MP);
-        *reinterpret_cast<uint2*>(dst) = make_uint2(sp[0], sp[1]);
-        if (full) {
-          const int64_t mbyte1 = mbyte0 + 8;
-          uint8_t* dst1 = meta + ((mbyte1 / MP) * m + gr) * MP + (mbyte1 % MP);
-          *reinterpret_cast<uint2*>(dst1) = make_uint2(sp[2], sp[3]);
-        }
+#pragma unroll
+        for (int w = 0; w < 4; w++)                      // one word per block of 32 columns; consecutive rows are adjacent
+          if (w < 2 || full) *reinterpret_cast<uint32_t*>(meta + panel_meta_offset(mbyte0 + 4 * w, gr, m)) = sp[w];
       }
     }
   }

@@ -37,7 +37,6 @@ prune_compress_dual(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t
   constexpr int TR = 128 / OS;                      // tile rows: the dense columns of one panel of W^T
   constexpr int TC = 128;                           // tile columns
   constexpr int UPP = (128 / OS) / 8;               // 8-element units per panel row
-  constexpr int MP = (128 / OS) / 8;                // metadata bytes per row per panel
   constexpr int KEEP = 8 * OS;                      // bit position of the keep flag in a tile element
   using E = std::conditional_t<OS == 2, uint32_t, uint16_t>;   // value bits | keep << KEEP
   constexpr int SW = 32 / (int)sizeof(E);           // columns per 32-byte swizzle unit
@@ -61,13 +60,14 @@ prune_compress_dual(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t
       const int lr = it * 16 + lr0;
       const int64_t row = row0 + lr;
       uint32_t mbyte = 0;
-      int64_t ounit = 0;
+      int64_t ounit = 0, ometa = 0;
       if (live) {
         Pack<In, 8> in;
         Pack<MaskT, 8> mk;
         in.load_stream(dense + row * ld + col8 * 8);
         mk.load_stream(mask + row * mask_ld + col8 * 8);
         ounit = panel ? ((col8 / UPP) * m + row) * UPP + col8 % UPP : row * upr + col8;
+        ometa = panel ? panel_meta_offset(col8, row, m) : ounit;
         Out cv[8];
         uint32_t keep = 0;
 #pragma unroll
@@ -94,7 +94,7 @@ prune_compress_dual(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t
       w |= __shfl_down(mbyte, 1) << 8;
       w |= __shfl_down(mbyte, 2) << 16;
       w |= __shfl_down(mbyte, 3) << 24;
-      if (live && (tid & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ounit) = w;
+      if (live && (tid & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ometa) = w;
     }
   }
   __syncthreads();
@@ -127,13 +127,25 @@ prune_compress_dual(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t
       const int64_t dst = panel ? ((gbyte >> 6) * k + trow) * 64 + (gbyte & 63) : trow * vrow_bytes + gbyte;
       o.store_stream(reinterpret_cast<Out*>(reinterpret_cast<uint8_t*>(values_t) + dst));
     }
-    // the 4 lanes of a column hold MP bytes of metadata between them: one panel row
+    // the 4 lanes of a column hold 8 (16) bytes of metadata between them: two (four) words of 32 columns
     const uint32_t b1 = __shfl_down(mbits, 1), b2 = __shfl_down(mbits, 2), b3 = __shfl_down(mbits, 3);
     if (live && q == 0) {
       const int64_t mbyte0 = row0 >> 3;
-      uint8_t* dst = panel ? meta_t + ((mbyte0 / MP) * k + trow) * MP : meta_t + trow * mrow_bytes + mbyte0;
-      if constexpr (OS == 2) *reinterpret_cast<uint2*>(dst) = make_uint2(mbits | (b1 << 16), b2 | (b3 << 16));
-      else *reinterpret_cast<uint4*>(dst) = make_uint4(mbits, b1, b2, b3);
+      if (panel) {
+        if constexpr (OS == 2) {
+          *reinterpret_cast<uint32_t*>(meta_t + panel_meta_offset(mbyte0, trow, k)) = mbits | (b1 << 16);
+          *reinterpret_cast<uint32_t*>(meta_t + panel_meta_offset(mbyte0 + 4, trow, k)) = b2 | (b3 << 16);
+        } else {
+          *reinterpret_cast<uint32_t*>(meta_t + panel_meta_offset(mbyte0, trow, k)) = mbits;
+          *reinterpret_cast<uint32_t*>(meta_t + panel_meta_offset(mbyte0 + 4, trow, k)) = b1;
+          *reinterpret_cast<uint32_t*>(meta_t + panel_meta_offset(mbyte0 + 8, trow, k)) = b2;
+          *reinterpret_cast<uint32_t*>(meta_t + panel_meta_offset(mbyte0 + 12, trow, k)) = b3;
+        }
+      } else {
+        uint8_t* dst = meta_t + trow * mrow_bytes + mbyte0;
+        if constexpr (OS == 2) *reinterpret_cast<uint2*>(dst) = make_uint2(mbits | (b1 << 16), b2 | (b3 << 16));
+        else *reinterpret_cast<uint4*>(dst) = make_uint4(mbits, b1, b2, b3);
+      }
     }
   }
 }

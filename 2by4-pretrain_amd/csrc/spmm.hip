@@ -153,12 +153,14 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
 #pragma unroll
     for (int ti = 0; ti < 2; ti++) {
       const int64_t row = i0 + ti * 16 + li;
-      // one instruction step is exactly one panel (KSTEP dense columns: 64 value bytes, KSTEP/8 metadata bytes)
+      // one instruction step is exactly one panel of values (KSTEP dense columns: 64 value bytes); the lane's
+      // index word is metadata bytes k0/8 + lk*2.. (16-bit values) or k0/8 + lk*4.. (8-bit) of its row
       const int64_t voff = panel ? ((k0 / KSTEP) * n_sparse + row) * 64 : row * a_pitch + (k0 / 2) * ES;
-      const int64_t moff = panel ? ((k0 / KSTEP) * n_sparse + row) * (KSTEP / 8) : row * m_pitch + k0 / 8;
+      const int64_t mbyte = k0 / 8 + lk * (ES == 2 ? 2 : 4);
+      const int64_t moff = panel ? panel_meta_offset(mbyte, row, n_sparse) : row * m_pitch + mbyte;
       af[ti] = *reinterpret_cast<const int4v*>(a_values + voff + lk * 16);
-      if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(a_meta + moff + lk * 2);
-      else idx[ti] = *reinterpret_cast<const int*>(a_meta + moff + lk * 4);
+      if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(a_meta + moff);
+      else idx[ti] = *reinterpret_cast<const int*>(a_meta + moff);
     }
     int8v bf[2];
 #pragma unroll
@@ -307,12 +309,12 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p) {
 // The source address is a wave-uniform 64-bit base in scalar registers plus a 32-bit offset per lane: with a
 // 64-bit address per lane the same copies hold up the matrix instructions issued around them (on an
 // instruction mix like the main loop's, 25 % more cycles than the matrix instructions alone against 3 %).
-__device__ __forceinline__ void g2l16(const uint8_t* base, uint32_t lane_offset, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
-}
 // same with one dword per lane: lane l writes LDS[base + 4*l]
 __device__ __forceinline__ void g2l4(const uint8_t* base, uint32_t lane_offset, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void g2l16(const uint8_t* base, uint32_t lane_offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
 }
 // s_waitcnt vmcnt(N) + s_barrier with a compile-time N (a bare s_barrier: __syncthreads() would add
 // a fence that drains every outstanding copy)
@@ -335,15 +337,22 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   constexpr int ES = sizeof(T);
   constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
   constexpr int M_STEP = M_ROW / C::STEPS;
-  // Metadata is copied one dword per lane (256 bytes per wave instruction) so that it can be laid
-  // out step-major in LDS, [step][row][M_STEP bytes]: the index words the 32 rows of a wave read for
-  // one step are then consecutive and conflict-free.  16-bit values: [step][row][4 bytes], a lane reads the
-  // halfword of its k half.  8-bit values (a dword per lane and k half): [step][k half][row][4 bytes], so
-  // that the 32 lanes of a half read 128 consecutive bytes -- row-major 8-byte entries put rows r and
-  // r + 16 of a 32-lane pass on one bank and every index read took two passes more.
+  // Metadata: in the panel form the words of 32 dense columns of consecutive rows are adjacent, [k/32][m][4 B],
+  // so the 256 rows of a tile are one 1 KB run per block of 32 columns and a stage is M_ROW/4 such runs (2 for
+  // 16-bit values, 4 for 8-bit ones).  In LDS they lie in the same order, [block][row][4 B], which is the order
+  // the index operands are read in: 16-bit values read the halfword of their k half from block = step; 8-bit
+  // values the dword of block = 2*step + k half; consecutive lanes read consecutive words either way.
+  // A run is one 16-byte-per-lane copy instruction; 8-bit values take those, issued by the last waves of the
+  // workgroup (copied a dword per lane, 16 instructions per stage, the same bytes took a fifth of the fp8
+  // kernel's copy time).  With 16-bit values and more waves than runs every wave brings a quarter run (or more)
+  // with dword copies instead, so that all waves run the same code: a branch in the loop body makes the compiler
+  // re-mask the 16-bit index words behind it, and that wait for all of a step's reads costs 5 %.
+  constexpr int STAGE_KB = M_ROW / 4;                        // 1 KB metadata runs per stage
+  constexpr bool M_DWORD = ES == 2 && C::NW > STAGE_KB;      // quarter runs, every wave
+  constexpr int MWAVES = M_DWORD ? C::NW : (STAGE_KB < C::NW ? STAGE_KB : C::NW);   // waves that copy metadata
+  constexpr int MW = (M_DWORD ? STAGE_KB * 4 : STAGE_KB) / MWAVES;                  // copies per such wave
+  static_assert(MW * MWAVES == (M_DWORD ? STAGE_KB * 4 : STAGE_KB) && C::BI * 4 == 1024, "metadata copies must divide among the waves");
   constexpr bool M_HALF_MAJOR = ES == 1;
-  constexpr int MW = C::BI * M_ROW / 256 / C::NW;           // dword copies per wave per stage (1 or 2)
-  static_assert(MW * 256 * C::NW == C::BI * M_ROW, "metadata copies must divide among the waves");
   // one stage buffer = [A values | B | A metadata]; three of them rotate
   constexpr int A_STAGE = C::BI * C::A_ROW, B_STAGE = C::BJ * C::B_ROW, M_STAGE = C::BI * M_ROW;
   constexpr int B_AT = A_STAGE, M_AT = A_STAGE + B_STAGE, STAGE_BYTES = A_STAGE + B_STAGE + M_STAGE;
@@ -407,7 +416,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     if constexpr (B_KSTRIDED) tile_b = b + (int64_t)st_begin * B_STAGE_ADVANCE_ROWS * ldb_bytes;   // columns stay absolute: the clamp may step left of the tile
     else tile_b = b + tj0 * ldb_bytes + (int64_t)st_begin * C::B_ROW;
     tile_a = a_values + (ti0 + (int64_t)st_begin * n_sparse) * 64;
-    tile_m = a_meta + (ti0 + (int64_t)st_begin * n_sparse) * M_ROW;
+    tile_m = a_meta + (ti0 + (int64_t)st_begin * STAGE_KB * n_sparse) * 4;
 #pragma unroll
     for (int q = 0; q < C::NB; q++) {
       if constexpr (B_KSTRIDED) {
@@ -429,23 +438,23 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     }
 #pragma unroll
     for (int q = 0; q < MW; q++) {
-      const int d = (wave * MW + q) * 64 + lane;               // dword index in the stage's step-major metadata
-      constexpr int DW_PER_STEP = C::BI * M_STEP / 4;
-      const int step = d / DW_PER_STEP, r = d % DW_PER_STEP;
-      const int row = M_HALF_MAJOR ? r % C::BI : r / (M_STEP / 4), part = M_HALF_MAJOR ? r / C::BI : r % (M_STEP / 4);
-      om[q] = (uint32_t)(min((int64_t)row, last_i) * M_ROW + step * M_STEP + part * 4);
+      const int c = (wave - (C::NW - MWAVES)) * MW + q;        // quarter run (a lane brings one row's word) or run (4 rows' words)
+      om[q] = M_DWORD ? (uint32_t)(((c >> 2) * n_sparse + min((int64_t)((c & 3) * 64 + lane), last_i)) * 4)
+                      : (uint32_t)((c * n_sparse + min((int64_t)lane * 4, last_i - 3)) * 4);
     }
   };
   point_at(i0, j0);
   const int64_t a_stage_stride = n_sparse * 64, m_stage_stride = n_sparse * M_ROW;
-  constexpr int NCOPY = C::NB + C::NA + MW;      // copies per wave per stage
+  constexpr int NCOPY = C::NB + C::NA + MW;      // copies per wave per stage (MW fewer for the waves without metadata)
+  const bool has_meta = MWAVES == C::NW || wave >= C::NW - MWAVES;      // the last waves (measured: 2.7 % better than the first ones at fp8)
 
   // copy q of this wave for stage st into the stage buffer at LDS byte address `dst`
   const uint32_t smem_at = lds_offset(smem);
   auto issue_one = [&](int q, int st, uint32_t dst) {
     if (q < C::NB) g2l16(tile_b + (int64_t)st * b_stage_stride, ob[q], dst + B_AT + (wave * C::NB + q) * 1024);
     else if (q < C::NB + C::NA) g2l16(tile_a + (int64_t)st * a_stage_stride, oa[q - C::NB], dst + (wave * C::NA + q - C::NB) * 1024);
-    else g2l4(tile_m + (int64_t)st * m_stage_stride, om[q - C::NB - C::NA], dst + M_AT + (wave * MW + q - C::NB - C::NA) * 256);
+    else if constexpr (M_DWORD) g2l4(tile_m + (int64_t)st * m_stage_stride, om[q - C::NB - C::NA], dst + M_AT + ((wave - (C::NW - MWAVES)) * MW + q - C::NB - C::NA) * 256);
+    else if (has_meta) g2l16(tile_m + (int64_t)st * m_stage_stride, om[q - C::NB - C::NA], dst + M_AT + ((wave - (C::NW - MWAVES)) * MW + q - C::NB - C::NA) * 1024);
   };
   auto issue = [&](int st, uint32_t dst) {
 #pragma unroll
@@ -571,7 +580,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   static_assert(!PERSIST || (C_JMAJOR && sizeof(OutT) == 2), "chained tiles rely on the wait inside the j-major 16-bit output pass");
   auto stage_barrier = [&](bool more) {          // B(st+1): only this wave's copies of stage st+2 may still fly
     if (!more) wait_copies_and_barrier<0>();
-    else wait_copies_and_barrier<NCOPY>();
+    else if (MWAVES == C::NW || has_meta) wait_copies_and_barrier<NCOPY>();
+    else wait_copies_and_barrier<NCOPY - MW>();
   };
 
   issue(0, smem_at);
@@ -961,7 +971,7 @@ spmm_narrow(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_
   const int64_t col = li < n_dense ? li : n_dense - 1;          // clamp: the column is never stored
   const uint8_t* bp = b + col * ldb_bytes + lk * 16;
   const uint8_t* av = a_values + (i0 + li) * 64 + lk * 16;
-  const uint8_t* am = a_meta + (i0 + li) * M_ROW + lk * (M_ROW / 4);
+  const uint8_t* am = a_meta + panel_meta_offset(lk * (M_ROW / 4), i0 + li, n_sparse);   // (a panel's further words: n_sparse * 4 bytes apart)
   const int64_t a_step = n_sparse * 64, m_step = n_sparse * M_ROW;
   acc_t acc[2];                              // two chains, so that consecutive instructions do not wait on each other
 #pragma unroll
@@ -1047,7 +1057,7 @@ spmm_narrow_shared(const uint8_t* __restrict__ a_values, const uint8_t* __restri
   const int64_t npanels = k / KSTEP;
   const int nchunks = (int)((npanels + CH - 1) / CH);
   const uint8_t* av = a_values + (i0 + li) * 64 + lk * 16;
-  const uint8_t* am = a_meta + (i0 + li) * M_ROW + lk * (M_ROW / 4);
+  const uint8_t* am = a_meta + panel_meta_offset(lk * (M_ROW / 4), i0 + li, n_sparse);   // (a panel's further words: n_sparse * 4 bytes apart)
   const int64_t a_step = n_sparse * 64, m_step = n_sparse * M_ROW;
   // dense chunk: thread's piece q = tid + THREADS j -> column q / (CH * 8), piece q % (CH * 8) of the column's 2 KB
   const uint8_t* bsrc[PIECES];

@@ -37,6 +37,12 @@ __host__ __device__ inline bool is_float8(int dt) { return dt == TF24_E4M3 || dt
 __host__ __device__ inline bool is_8bit(int dt) { return is_float8(dt) || dt == TF24_I8; }
 template <> struct dtype_of<uint8_t> { static constexpr int value = TF24_U8; };
 
+// Panel form of the metadata, [k/32][m][4 bytes]: byte offset of metadata byte `mbyte` (= dense column / 8)
+// of row `row` of a matrix with m rows.
+__host__ __device__ inline int64_t panel_meta_offset(int64_t mbyte, int64_t row, int64_t m) {
+  return ((mbyte >> 2) * m + row) * 4 + (mbyte & 3);
+}
+
 __host__ __device__ inline int dtype_size(int dt) {
   return (dt == TF24_F32 || dt == TF24_I32) ? 4 : (dt == TF24_F16 || dt == TF24_BF16) ? 2 : 1;
 }

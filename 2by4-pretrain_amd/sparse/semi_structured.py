@@ -60,7 +60,7 @@ def _to_canonical(values, meta, m, n):
     """Panel-layout storage -> canonical (values [m, n/2], meta [m, n/16 | n/32])."""
     kp = _panel_width(values.dtype)
     v = values.view(n // kp, m, kp // 2).permute(1, 0, 2).reshape(m, n // 2)
-    mt = meta.view(n // kp, m, 4).permute(1, 0, 2).reshape(m, -1)
+    mt = meta.view(n // 32, m, 4 // meta.element_size()).permute(1, 0, 2).reshape(m, -1)   # [n/32][m][4 bytes] -> rows
     return v, mt
 
 
@@ -435,7 +435,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
     def indices_cutlass(self):
         """Metadata in the CUTLASS-reordered layout the reference's `indices()` returns
         (reorder_meta + ColumnMajorInterleaved<2>; csrc .cu:826-851)."""
-        meta = self.meta_tensor_cutlass
+        meta = self.meta_tensor_cutlass.contiguous()
         m, ncols = meta.shape
         group, inter = (32, 4) if meta.dtype == torch.int16 else (16, 2)
         r = torch.arange(m, device=meta.device).view(-1, 1).expand(m, ncols)

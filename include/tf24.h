@@ -67,12 +67,14 @@ typedef enum { TF24_ACT_NONE = 0, TF24_ACT_RELU = 1, TF24_ACT_SILU = 2, TF24_ACT
 /*
  * Storage of a compressed [m,k] matrix (values + metadata).
  *   CANONICAL  values [m, k/2] row-major, metadata [m, k/8 bytes] row-major (the interchange form).
- *   PANEL      the SMFMAC-native form the matmul streams: the k axis is cut into panels of
- *              KP = 128/sizeof(value) dense columns (64 for 16-bit values, 128 for fp8), i.e. the
- *              64 value bytes and KP/8 metadata bytes one row contributes to one LDS stage;
- *              values [k/KP][m][64 bytes], metadata [k/KP][m][KP/8 bytes].  A 256-row tile of one
- *              stage is then a single contiguous 16 KB (+2/4 KB) run, copied to LDS with full-line
- *              GLOBAL_LOAD_LDS_DWORDX4.  Inside a row of a panel the bytes are the canonical ones.
+ *   PANEL      the SMFMAC-native form the matmul streams.  Values: the k axis is cut into panels of
+ *              KP = 128/sizeof(value) dense columns (64 for 16-bit values, 128 for 8-bit ones), i.e. the
+ *              64 value bytes one row contributes to one LDS stage: [k/KP][m][64 bytes], the bytes of a
+ *              row inside a panel being the canonical ones.  Metadata: the 4-byte word of 32 dense
+ *              columns (8 nibbles, canonical order) of every row, column-block-major: [k/32][m][4 bytes].
+ *              A 256-row tile of one stage is then one contiguous 16 KB run of values and 2 (4) contiguous
+ *              1 KB runs of metadata, all copied to LDS with full-line GLOBAL_LOAD_LDS_DWORDX4, and the
+ *              metadata lands in the order the matrix instructions' index operands are read in.
  */
 typedef enum { TF24_COMPRESSED_CANONICAL = 0, TF24_COMPRESSED_PANEL = 1 } tf24_compressed_layout;
 
