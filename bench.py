@@ -1,6 +1,6 @@
 """Benchmark of the 2:4 sparse hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|train|fp8|decode|traffic] [--no-cpu] [--no-convert] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload spmm|train|fp8|int8|decode|traffic] [--no-cpu] [--no-convert] [--no-extra]
 
 Default workload: BASELINE config 3 -- fp16 2:4 spMM forward  Y[8192,11008] = X[8192,4096] . W^T
 (W[11008,4096] magnitude-pruned along K) plus the transposed product dX[8192,4096] = dY . W with
@@ -298,6 +298,41 @@ def train_workload(steps, warmup):
     return sparse_ms, dense_ms, sparse_loss, dense_loss, flops, one_pass_ms
 
 
+def int8_workload(steps):
+    """Not a BASELINE config (the reference's int8 branch, csrc .cu:594-637): int8 A[16384,8192] x magnitude-pruned
+    int8 B[8192,8192]^T, int32 accumulate and output; comparator torch._int_mm on the dense masked operand.
+    Exact: checked against an int64 product on a slab of rows."""
+    import sparse
+    dev = torch.device("cuda:0")
+    M, K, Nb = 16384, 8192, 8192
+    gen = torch.Generator(device=dev).manual_seed(7)
+    A = torch.randint(-127, 128, (M, K), device=dev, generator=gen, dtype=torch.int32).to(torch.int8)
+    B = torch.randint(-127, 128, (Nb, K), device=dev, generator=gen, dtype=torch.int32).to(torch.int8)
+    w = sparse.to_sparse_semi_structured(B, dtype=torch.int8)
+    Bd = w.to_dense()
+    del B
+
+    def timed(fn):
+        settle(lambda i: fn())
+        e = _events(2)
+        e[0].record()
+        for _ in range(steps):
+            fn()
+        e[1].record()
+        torch.cuda.synchronize()
+        return e[0].elapsed_time(e[1]) / steps
+
+    mm_ms = timed(lambda: torch.mm(A, w.t()))
+    dense_ms = None
+    try:
+        dense_ms = timed(lambda: torch._int_mm(A, Bd.t()))
+    except Exception as ex:
+        print(f"bench.py: dense int8 comparator unavailable: {ex}", file=sys.stderr)
+    rows = slice(0, 256)
+    exact = bool(torch.mm(A[rows], w.t()).cpu().long().equal(A[rows].cpu().long() @ Bd.cpu().long().t()))
+    return mm_ms, dense_ms, exact, 2.0 * M * K * Nb
+
+
 def fp8_workload(steps, warmup):
     """BASELINE configs[4]: e4m3 2:4 spMM A[16384,8192] x B[8192,8192]^T with B MVUE24-pruned from seeded
     uniforms, bf16 output; one step = soft_threshold24 on the bf16 B + MVUE24 prune/compress to e4m3 +
@@ -513,7 +548,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["spmm", "train", "fp8", "decode", "traffic"], default="spmm",
+    ap.add_argument("--workload", choices=["spmm", "train", "fp8", "int8", "decode", "traffic"], default="spmm",
                     help="spmm: BASELINE configs[2] (default, the judged line); train: configs[3] MLP training step; "
                          "fp8: configs[4] e4m3 MVUE + spMM; decode: 8-1024 tokens against the config-3 weight (not a BASELINE config); "
                          "traffic: kernels of known footprint + the config-3 products, for rocprofv3 --pmc byte-counter runs")
@@ -557,6 +592,21 @@ def main():
             "roofline": {"bound": "hbm", "kernel": "spmm_narrow_shared (8 tokens)", "achieved": first["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": first["frac_of_hbm_peak"], "traffic": None},
             "by_tokens": rows, "cpu_baseline": None}))
+        return
+
+    if a.workload == "int8":
+        mm_ms, dense_ms, exact, ops = int8_workload(a.steps)
+        executed = (ops / 2) / (mm_ms * 1e-3) / 1e12
+        print(json.dumps({
+            "metric": "int8 2:4 spMM TOP/s (dense-equivalent 2MNK)", "value": round(ops / (mm_ms * 1e-3) / 1e12, 2),
+            "unit": "TOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_s": SETTLE_S, "ms_per_step": round(mm_ms, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+            "config": {"workload": "not a BASELINE config: int8 A[16384,8192] x magnitude-pruned int8 B[8192,8192]^T, int32 accumulate and output", "seed": 7},
+            "roofline": {"bound": "mfma", "kernel": "spmm (SMFMAC int8)", "achieved": round(executed, 2), "peak": 5000.0, "unit": "TOP/s",
+                         "frac": round(executed / 5000.0, 4), "traffic": None},
+            "dense_int8_gemm_ms": None if dense_ms is None else round(dense_ms, 4),
+            "speedup_vs_dense_gemm": None if dense_ms is None else round(dense_ms / mm_ms, 3),
+            "exact_vs_int64_product": exact, "cpu_baseline": None}))
         return
 
     if a.workload == "fp8":
