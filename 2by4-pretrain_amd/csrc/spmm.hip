@@ -1325,7 +1325,8 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout,
   if (rc) return rc;
   if (!a_values || !a_meta || !b || !c) return fail(TF24_ERR_ARG, "tf24_spmm: null pointer");
   if ((rc = check_aligned("tf24_spmm", 16, {a_values, b, c, workspace}))) return rc;
-  if ((rc = check_aligned("tf24_spmm", 8, {a_meta}))) return rc;
+  // panel metadata is copied 16 bytes per lane; canonical metadata is read in words of up to 4 bytes, row pitch k/8
+  if ((rc = check_aligned("tf24_spmm", a_layout == TF24_COMPRESSED_PANEL ? 16 : 8, {a_meta}))) return rc;
   if ((rc = check_aligned("tf24_spmm", dtype_size(out_dtype), {bias}))) return rc;
   if (a_layout != TF24_COMPRESSED_CANONICAL && a_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_spmm: bad compressed layout %d", a_layout);
   const bool panel = a_layout == TF24_COMPRESSED_PANEL;

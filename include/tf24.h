@@ -300,7 +300,8 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * Shape rules (.cu:101-109): n_sparse % 32 == 0, k % 64 == 0 (16-bit) / 128 (8-bit),
  * n_dense % 8 == 0 (16-bit) / 16 (8-bit).  Leading dimensions: ldb a multiple of 8 (16-bit) / 16 (8-bit)
  * elements and at most 16 MiB per row (a tile's rows are addressed by 32-bit offsets), ldc a multiple of 8 for
- * 16-bit outputs and of 4 for 32-bit ones (16-byte row segments); b, c, a_values 16-byte aligned.
+ * 16-bit outputs and of 4 for 32-bit ones (16-byte row segments); b, c, a_values 16-byte aligned, a_meta 16-byte
+ * aligned in panel form (8 in canonical form).
  */
 int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,
               const void* b, int b_layout, int64_t ldb, int64_t n_dense,
