@@ -674,6 +674,27 @@ def test_transpose_copy(cuda, dtype, shape):
     assert_same(out, t.t().contiguous())
 
 
+@pytest.mark.parametrize("dtype", [F16, E4M3, torch.int8])
+def test_panel_form_is_the_documented_one(cuda, dtype):
+    """The panel form as the C header states it, spelled out with torch views of the canonical tensors:
+    values [k/KP][m][64 bytes] (KP = 128 / sizeof(value) dense columns), metadata [k/32][m][4 bytes]."""
+    import sparse
+    from sparse import _native as N
+    m, k = 96, 640
+    if dtype == torch.int8:
+        w = torch.randint(-100, 101, (m, k), generator=torch.Generator().manual_seed(93)).to(torch.int8)
+    else:
+        w = randn((m, k), F32, 92)
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    assert s._store_layout == N.COMPRESSED_PANEL
+    want_v, want_m = oracle.compress24(w, out_dtype=dtype)
+    kp = 128 // want_v.element_size()
+    v_bytes = want_v.contiguous().view(torch.uint8).reshape(m, k // kp, 64).permute(1, 0, 2).contiguous()
+    m_bytes = want_m.contiguous().view(torch.uint8).reshape(m, k // 32, 4).permute(1, 0, 2).contiguous()
+    assert s._store_values.contiguous().view(torch.uint8).cpu().reshape(k // kp, m, 64).equal(v_bytes)
+    assert s._store_meta.contiguous().view(torch.uint8).cpu().reshape(k // 32, m, 4).equal(m_bytes)
+
+
 @pytest.mark.parametrize("dtype", [F16, E4M3])
 def test_repack_between_canonical_and_panel(cuda, dtype):
     """tf24_repack on canonical values/metadata must give the bytes the compress kernel writes in
