@@ -89,7 +89,14 @@ __host__ __device__ inline uint8_t float_to_e4m3(float f) {
   }
   return (uint8_t)(r | sign);
 }
-template <> __device__ __forceinline__ e4m3_t from_float<e4m3_t>(float f) { return e4m3_t{float_to_e4m3(f)}; }
+// On the device gfx950's V_CVT_PK_FP8_F32 (OCP e4m3fn, round to nearest even, NaN past the range) gives the same
+// byte for every float32 pattern that is not a NaN; NaNs take the bit arithmetic's sign | 0x7f (the instruction
+// returns 0xff for both signs).  About five instructions instead of twenty.
+template <> __device__ __forceinline__ e4m3_t from_float<e4m3_t>(float f) {
+  const uint32_t h = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false) & 0xffu;
+  const uint32_t nan = ((__builtin_bit_cast(uint32_t, f) >> 24) & 0x80u) | 0x7fu;
+  return e4m3_t{(uint8_t)(f != f ? nan : h)};
+}
 
 __host__ __device__ inline float e4m3_to_float(uint8_t b) {
   uint32_t sign = (uint32_t)(b & 0x80u) << 24;
@@ -122,7 +129,12 @@ __host__ __device__ inline uint8_t float_to_e5m2(float f) {
   }
   return (uint8_t)(r | sign);
 }
-template <> __device__ __forceinline__ e5m2_t from_float<e5m2_t>(float f) { return e5m2_t{float_to_e5m2(f)}; }
+// V_CVT_PK_BF8_F32: as above (its NaN is 0x7e | sign; the bit arithmetic's, and torch's, 0x7f | sign)
+template <> __device__ __forceinline__ e5m2_t from_float<e5m2_t>(float f) {
+  const uint32_t h = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(f, f, 0, false) & 0xffu;
+  const uint32_t nan = ((__builtin_bit_cast(uint32_t, f) >> 24) & 0x80u) | 0x7fu;
+  return e5m2_t{(uint8_t)(f != f ? nan : h)};
+}
 // int8: exact for the integers an int8 dense operand holds (the only input the int8 path accepts)
 template <> __device__ __forceinline__ i8_t from_float<i8_t>(float f) {
   const float c = f < -128.0f ? -128.0f : (f > 127.0f ? 127.0f : f);
