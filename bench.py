@@ -29,12 +29,12 @@ MFMA_DENSE_PEAK_FP8_TFLOPS = 5000.0
 # Bytes that cross the L2 <-> memory-fabric boundary per spmm launch of config 3 (mean of forward and
 # transposed), from two `rocprofv3 --pmc` runs of `bench.py --workload traffic` (FETCH_SIZE, then
 # WRITE_SIZE; KiB per dispatch), each scaled by known / counted bytes of a plain 128 MiB device copy in
-# the same run: FETCH_SIZE 422604 KiB x 2.00 (the counter books this GPU's 128-byte read requests as 64
+# the same run: FETCH_SIZE 431052 KiB x 2.00 (the counter books this GPU's 128-byte read requests as 64
 # bytes: every streaming kernel of known footprint reads 0.50 of its bytes, and the 32-byte-unit request
-# counter TCC_EA0_RDREQ_DRAM_32B gives 856 MB against 865), WRITE_SIZE 120847 KiB x 1.00.  The infinity
+# counter TCC_EA0_RDREQ_DRAM_32B gives the same 883 MB), WRITE_SIZE 120841 KiB x 1.00.  The infinity
 # cache sits behind this boundary, so part of it never reaches HBM.  A profiled constant, not
 # something this run measures: emitted for the config-3 shape only, with its source.
-SPMM_TRAFFIC_PROFILED = int(422604 * 1024 * 2.0 + 120847 * 1024 * 1.0)
+SPMM_TRAFFIC_PROFILED = int(431052 * 1024 * 2.0 + 120841 * 1024 * 1.0)
 SPMM_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over `bench.py --workload traffic`, factors 2.00 / 1.00 from the "
                        "128 MiB device copy of the same runs; L2 <-> fabric bytes (infinity cache behind it); summary under profiles/")
 
