@@ -129,8 +129,9 @@ template <typename T, typename OutT, bool B_KCONTIG, bool C_JMAJOR>
 __global__ void __launch_bounds__(256)
 spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
              const T* __restrict__ b, int64_t ldb, int64_t n_dense,
-             OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act, bool panel) {
+             OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act, int a_layout) {
   constexpr int KSTEP = mma16<T>::KSTEP;
+  const bool panel = a_layout == TF24_COMPRESSED_PANEL;
   constexpr int ES = sizeof(T);                       // element size of values and B
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t i0 = (int64_t)blockIdx.y * 64 + (wave >> 1) * 32;
@@ -138,7 +139,6 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
   if (i0 >= n_sparse || j0 >= n_dense) return;       // whole wave out of range
   const int li = lane & 15, lk = lane >> 4;
   const int64_t a_pitch = (k / 2) * ES;               // bytes per row of compressed values
-  const int64_t m_pitch = k / 8;                      // bytes per row of metadata
   typename mma16<T>::acc_t acc[2][2];
 #pragma unroll
   for (int ti = 0; ti < 2; ti++)
@@ -157,7 +157,7 @@ spmm_general(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a
       // index word is metadata bytes k0/8 + lk*2.. (16-bit values) or k0/8 + lk*4.. (8-bit) of its row
       const int64_t voff = panel ? ((k0 / KSTEP) * n_sparse + row) * 64 : row * a_pitch + (k0 / 2) * ES;
       const int64_t mbyte = k0 / 8 + lk * (ES == 2 ? 2 : 4);
-      const int64_t moff = panel ? panel_meta_offset(mbyte, row, n_sparse) : row * m_pitch + mbyte;
+      const int64_t moff = meta_offset<ES == 2 ? 2 : 4>(a_layout, mbyte, row, n_sparse, k);   // (reordered metadata: the reference's own storage)
       af[ti] = *reinterpret_cast<const int4v*>(a_values + voff + lk * 16);
       if constexpr (ES == 2) idx[ti] = *reinterpret_cast<const uint16_t*>(a_meta + moff);
       else idx[ti] = *reinterpret_cast<const int*>(a_meta + moff);
@@ -1180,13 +1180,13 @@ int launch_narrow(const void* av, const void* am, int64_t n_sparse, int64_t k, c
 }
 
 template <typename T, typename OutT>
-int launch_general(const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
+int launch_general(const void* av, const void* am, int a_layout, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                    int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act, hipStream_t s) {
   dim3 grid((unsigned)((n_dense + 63) / 64), (unsigned)((n_sparse + 63) / 64));
   const bool kc = b_layout == TF24_ROW_MAJOR, jm = c_layout == TF24_COL_MAJOR;
 #define TF24_GO(KC, JM)                                                                                              \
   hipLaunchKernelGGL((spmm_general<T, OutT, KC, JM>), grid, dim3(256), 0, s, (const uint8_t*)av, (const uint8_t*)am, \
-                     n_sparse, k, (const T*)b, ldb, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, panel)
+                     n_sparse, k, (const T*)b, ldb, n_dense, (OutT*)c, ldc, (const OutT*)bias, scale, act, a_layout)
   if (kc && jm) TF24_GO(true, true);
   else if (kc) TF24_GO(true, false);
   else if (jm) TF24_GO(false, true);
@@ -1196,9 +1196,10 @@ int launch_general(const void* av, const void* am, bool panel, int64_t n_sparse,
 }
 
 template <typename T>
-int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int64_t n_sparse, int64_t k, const void* b, int b_layout,
+int dispatch_out(int out_dtype, const void* av, const void* am, int a_layout, int64_t n_sparse, int64_t k, const void* b, int b_layout,
                  int64_t ldb, int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  void* workspace, int64_t workspace_bytes, hipStream_t s) {
+  const bool panel = a_layout == TF24_COMPRESSED_PANEL;
   // the tiled kernel reads a k-strided dense operand through transposing LDS reads (16-bit types only)
   // (also for a narrow dense operand: with its k pieces the tiled kernel beats the general one from 8 columns on)
   const bool tiled = panel && (b_layout == TF24_ROW_MAJOR || sizeof(T) == 2) && n_sparse >= 64;
@@ -1221,7 +1222,7 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
     if (slim) return launch_tiled<T, int32_t, SlimCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     if (mid) return launch_tiled<T, int32_t, MidCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
     if (tiled) return launch_tiled<T, int32_t, TiledCfg>(av, am, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, workspace, workspace_bytes, s);
-    return launch_general<T, int32_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    return launch_general<T, int32_t>(av, am, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   } else {
   if (narrow) {
     switch (out_dtype) {
@@ -1252,9 +1253,9 @@ int dispatch_out(int out_dtype, const void* av, const void* am, bool panel, int6
     }
   }
   switch (out_dtype) {
-    case TF24_F16: return launch_general<T, f16_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-    case TF24_BF16: return launch_general<T, bf16_t>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
-    case TF24_F32: return launch_general<T, float>(av, am, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_F16: return launch_general<T, f16_t>(av, am, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_BF16: return launch_general<T, bf16_t>(av, am, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
+    case TF24_F32: return launch_general<T, float>(av, am, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, act, s);
   }
   return fail(TF24_ERR_DTYPE, "tf24_spmm: unsupported output dtype %d", out_dtype);
   }
@@ -1326,17 +1327,17 @@ extern "C" int tf24_spmm(const void* a_values, const void* a_meta, int a_layout,
   if (!a_values || !a_meta || !b || !c) return fail(TF24_ERR_ARG, "tf24_spmm: null pointer");
   if ((rc = check_aligned("tf24_spmm", 16, {a_values, b, c, workspace}))) return rc;
   // panel metadata is copied 16 bytes per lane; canonical metadata is read in words of up to 4 bytes, row pitch k/8
-  if ((rc = check_aligned("tf24_spmm", a_layout == TF24_COMPRESSED_PANEL ? 16 : 8, {a_meta}))) return rc;
+  if ((rc = check_aligned("tf24_spmm", a_layout == TF24_COMPRESSED_PANEL ? 16 : a_layout == TF24_COMPRESSED_CUTLASS ? 4 : 8, {a_meta}))) return rc;
   if ((rc = check_aligned("tf24_spmm", dtype_size(out_dtype), {bias}))) return rc;
-  if (a_layout != TF24_COMPRESSED_CANONICAL && a_layout != TF24_COMPRESSED_PANEL) return fail(TF24_ERR_ARG, "tf24_spmm: bad compressed layout %d", a_layout);
-  const bool panel = a_layout == TF24_COMPRESSED_PANEL;
+  if (a_layout != TF24_COMPRESSED_CANONICAL && a_layout != TF24_COMPRESSED_PANEL && a_layout != TF24_COMPRESSED_CUTLASS)
+    return fail(TF24_ERR_ARG, "tf24_spmm: bad compressed layout %d", a_layout);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == TF24_I8 && scale != 1.0f) return fail(TF24_ERR_ARG, "tf24_spmm: int8 products are exact, scale must be 1 (%g given)", (double)scale);
   switch (dtype) {
-    case TF24_I8: return dispatch_out<i8_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
-    case TF24_E5M2: return dispatch_out<e5m2_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
-    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, panel, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    case TF24_I8: return dispatch_out<i8_t>(out_dtype, a_values, a_meta, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    case TF24_F16: return dispatch_out<f16_t>(out_dtype, a_values, a_meta, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, a_values, a_meta, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    case TF24_E5M2: return dispatch_out<e5m2_t>(out_dtype, a_values, a_meta, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
+    default: return dispatch_out<e4m3_t>(out_dtype, a_values, a_meta, a_layout, n_sparse, k, b, b_layout, ldb, n_dense, c, c_layout, ldc, bias, scale, activation, workspace, workspace_bytes, s);
   }
 }

@@ -43,6 +43,28 @@ __host__ __device__ inline int64_t panel_meta_offset(int64_t mbyte, int64_t row,
   return ((mbyte >> 2) * m + row) * 4 + (mbyte & 3);
 }
 
+// CUTLASS form of the metadata (reorder_meta + ColumnMajorInterleaved<2>, reference csrc .cu:826-851):
+// byte offset of metadata byte `mbyte` of row `row`.  WB = bytes per metadata word (2: int16 words of
+// 16-bit values, 4: int32 words of 8-bit values).  Word (row, c) moves to row
+// row/G*G + (row%8)*I + (row%G)/8 with (G, I) = (32, 4) | (16, 2), is swapped inside 2 x 2 blocks (even
+// row, odd column <-> odd row, even column) and lands at word (c'/2)*2m + 2*row' + c'%2.
+template <int WB>
+__host__ __device__ inline int64_t cutlass_meta_offset(int64_t mbyte, int64_t row, int64_t m) {
+  constexpr int G = WB == 2 ? 32 : 16, I = WB == 2 ? 4 : 2;
+  const int64_t c = mbyte / WB;
+  int64_t dr = row / G * G + (row % 8) * I + (row % G) / 8, dc = c;
+  if ((dr & 1) == 0 && (dc & 1) == 1) { dr++; dc--; }
+  else if ((dr & 1) == 1 && (dc & 1) == 0) { dr--; dc++; }
+  return ((dc >> 1) * m * 2 + dr * 2 + (dc & 1)) * WB + mbyte % WB;
+}
+// byte offset of metadata byte `mbyte` of row `row` in any of the three storage forms (k = dense columns)
+template <int WB>
+__host__ __device__ inline int64_t meta_offset(int layout, int64_t mbyte, int64_t row, int64_t m, int64_t k) {
+  if (layout == TF24_COMPRESSED_PANEL) return panel_meta_offset(mbyte, row, m);
+  if (layout == TF24_COMPRESSED_CUTLASS) return cutlass_meta_offset<WB>(mbyte, row, m);
+  return row * (k >> 3) + mbyte;
+}
+
 __host__ __device__ inline int dtype_size(int dt) {
   return (dt == TF24_F32 || dt == TF24_I32) ? 4 : (dt == TF24_F16 || dt == TF24_BF16) ? 2 : 1;
 }

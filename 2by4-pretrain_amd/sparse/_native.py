@@ -16,7 +16,7 @@ F32, F16, BF16, E4M3, U8, E5M2, I8, I32 = 0, 1, 2, 3, 4, 5, 6, 7
 ROW_MAJOR, COL_MAJOR = 0, 1
 PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE, PRUNE_MVUE_PACKED, PRUNE_MVUE_SEEDED = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
-COMPRESSED_CANONICAL, COMPRESSED_PANEL = 0, 1
+COMPRESSED_CANONICAL, COMPRESSED_PANEL, COMPRESSED_CUTLASS = 0, 1, 2
 
 _DTYPES = {
     torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float8_e4m3fn: E4M3, torch.float8_e5m2: E5M2,
@@ -43,6 +43,7 @@ _SIGNATURES = {
     "tf24_prune_compress_dual_validate": (_i, [_i, _i64, _i64, _i64, _i, _i64, _i, _i]),
     "tf24_decompress": (_i, [_p, _i, _p, _i, _i64, _i64, _p, _p]),
     "tf24_repack": (_i, [_p, _p, _i, _i64, _i64, _i, _p, _p, _p]),
+    "tf24_repack_to": (_i, [_p, _p, _i, _i64, _i64, _i, _i, _p, _p, _p]),
     "tf24_transposable_mask": (_i, [_p, _i, _i, _i64, _i64, _i64, _i, _p, _p, _p]),
     "tf24_transposable_mask_validate": (_i, [_i, _i, _i64, _i64, _i64]),
     "tf24_soft_threshold24": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _p, _p]),

@@ -9,8 +9,10 @@ behaviour.  Differences, all deliberate:
     TF24_COMPRESSED_PANEL; class flag `_PANEL_LAYOUT`); `values()` / `indices()` /
     `sparse_tensor_cutlass` / `meta_tensor_cutlass` materialise the canonical row-major form
     (values [m, k/2], nibble metadata [m, k/16 | k/32]) on first use, also for column-major
-    inputs (`W.T`); the metadata is the canonical nibble stream, not CUTLASS's reordered layout --
-    `indices_cutlass()` exports the reordered form;
+    inputs (`W.T`); the metadata is the canonical nibble stream by default, and CUTLASS's reordered
+    layout -- what the reference stores, returns from `indices()` and takes as `meta_tensor_cutlass=`
+    (semi_structured.py:536-546, :133-144) -- when the class flag `_CUTLASS_METADATA` is set;
+    `indices_cutlass()` / `indices_canonical()` give either form regardless of the flag;
   * MVUE24 takes its uniforms from an optional `rand` tensor, or generates them inside the kernel from
     (seed, offset) -- `rand=(seed, offset)`, or torch's generator state when `rand` is omitted;
   * `addmm` / `linear` with a bias work (the reference passes a wrong keyword there).
@@ -151,18 +153,22 @@ def _compress(original, dtype, MVUE24, mask, rand, panel, row_sums=False):
 _WORKSPACE_BYTES = {}      # (dtype, n, k, j) -> tf24_spmm_workspace_bytes, a pure function of the shape
 
 
-def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, activation=N.ACT_NONE):
+def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, activation=N.ACT_NONE, keep_panel=True):
     """sparse_first: out = S @ dense  (S [n,k], dense [k,j])  -> [n, j]
-       otherwise   : out = dense @ S^T (dense [j,k])          -> [j, n]"""
+       otherwise   : out = dense @ S^T (dense [j,k])          -> [j, n]
+    keep_panel: an operand that arrives in canonical or CUTLASS form is repacked to the panel form; keep
+    that copy in the wrapper (the wrapper owns its tensors) or drop it after the product (the wrapper
+    only borrows tensors its caller may rewrite)."""
     values, meta, store_layout = sparse._store_values, sparse._store_meta, sparse._store_layout
     n, k = sparse._store_shape
     # An operand built from canonical values/metadata (the functional entry point) is brought to the
     # panel form once: the tiled kernel only streams that one.
-    if store_layout == N.COMPRESSED_CANONICAL and n >= 64 and k % _panel_width(values.dtype) == 0:
+    if store_layout != N.COMPRESSED_PANEL and n >= 64 and k % _panel_width(values.dtype) == 0:
         pv, pm = torch.empty_like(values), torch.empty_like(meta)
-        N.check(N.lib().tf24_repack(values.data_ptr(), meta.data_ptr(), N.operand_code(values.dtype), n, k, N.COMPRESSED_CANONICAL,
-                                    pv.data_ptr(), pm.data_ptr(), N.stream_ptr()))
-        sparse._set_storage(pv, pm, (n, k), N.COMPRESSED_PANEL)
+        N.check(N.lib().tf24_repack_to(values.data_ptr(), meta.data_ptr(), N.operand_code(values.dtype), n, k, store_layout,
+                                       N.COMPRESSED_PANEL, pv.data_ptr(), pm.data_ptr(), N.stream_ptr()))
+        if keep_panel:
+            sparse._set_storage(pv, pm, (n, k), N.COMPRESSED_PANEL)
         values, meta, store_layout = pv, pm, N.COMPRESSED_PANEL
     if dense.dtype != values.dtype:
         raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
@@ -241,6 +247,11 @@ class SparseSemiStructuredTensor(torch.Tensor):
     _FP8_OUT_DTYPE = torch.float32
     # store freshly compressed tensors in the SMFMAC panel layout (False: canonical row-major)
     _PANEL_LAYOUT = True
+    # True: `indices()` / `meta_tensor_cutlass` return, and the `meta_tensor_cutlass=` constructor argument
+    # is read as, the CUTLASS-reordered metadata of the reference (semi_structured.py:536-546; csrc
+    # .cu:826-851) instead of the canonical nibble stream.  Set it before building tensors whose
+    # metadata is exchanged with code written against the reference or upstream torch.sparse.
+    _CUTLASS_METADATA = False
 
     @staticmethod
     def __new__(cls, original_tensor: Optional[torch.Tensor], original_shape: Optional[torch.Size] = None,
@@ -296,10 +307,11 @@ class SparseSemiStructuredTensor(torch.Tensor):
             values, meta = _compress(original_tensor, dtype, MVUE24, mask, rand, panel)
             self._set_storage(values, meta, (m, n), N.COMPRESSED_PANEL if panel else N.COMPRESSED_CANONICAL)
         elif sparse_tensor_cutlass is not None:
-            # built from canonical pieces (values [m, k/2], nibble metadata)
+            # built from pieces: values [m, k/2] row-major and metadata, canonical nibble stream or (class
+            # flag) the reference's reordered words
             mm, half = sparse_tensor_cutlass.shape
             self._set_storage(sparse_tensor_cutlass.contiguous().view(-1), meta_tensor_cutlass.contiguous().view(-1),
-                              (mm, 2 * half), N.COMPRESSED_CANONICAL)
+                              (mm, 2 * half), N.COMPRESSED_CUTLASS if self._CUTLASS_METADATA else N.COMPRESSED_CANONICAL)
         else:
             self._set_storage(None, None, None, N.COMPRESSED_CANONICAL)
         self.original_tensor = None
@@ -311,15 +323,32 @@ class SparseSemiStructuredTensor(torch.Tensor):
         self._store_values, self._store_meta = values, meta       # flat device tensors
         self._store_shape, self._store_layout = shape, layout     # (m, k) of the untransposed matrix
         self._canonical = None
+        self._cutlass = None
 
     def _canonical_pair(self):
         if self._canonical is None:
             m, n = self._store_shape
             if self._store_layout == N.COMPRESSED_PANEL:
                 self._canonical = _to_canonical(self._store_values, self._store_meta, m, n)
+            elif self._store_layout == N.COMPRESSED_CUTLASS:
+                self._canonical = (self._store_values.view(m, n // 2), self._converted_meta(N.COMPRESSED_CANONICAL))
             else:
                 self._canonical = (self._store_values.view(m, n // 2), self._store_meta.view(m, -1))
         return self._canonical
+
+    def _converted_meta(self, to_layout):
+        """The metadata in another storage form, [m, k/16 | k/32] words (HIP kernel; values untouched)."""
+        m, n = self._store_shape
+        out = torch.empty_like(self._store_meta)
+        if self._store_layout == N.COMPRESSED_PANEL:
+            # only the metadata is wanted: go through the canonical view of the panel words
+            src = self._canonical_pair()[1].contiguous()
+            N.check(N.lib().tf24_repack_to(None, src.data_ptr(), N.operand_code(self._store_values.dtype), m, n,
+                                           N.COMPRESSED_CANONICAL, to_layout, None, out.data_ptr(), N.stream_ptr()))
+        else:
+            N.check(N.lib().tf24_repack_to(None, self._store_meta.data_ptr(), N.operand_code(self._store_values.dtype), m, n,
+                                           self._store_layout, to_layout, None, out.data_ptr(), N.stream_ptr()))
+        return out.view(m, -1)
 
     @property
     def sparse_tensor_cutlass(self):
@@ -328,8 +357,11 @@ class SparseSemiStructuredTensor(torch.Tensor):
 
     @property
     def meta_tensor_cutlass(self):
-        """Canonical nibble metadata [m, k/16] int16 or [m, k/32] int32."""
-        return None if self._store_values is None else self._canonical_pair()[1]
+        """Metadata [m, k/16] int16 or [m, k/32] int32: the canonical nibble stream, or with the class flag
+        `_CUTLASS_METADATA` the reference's reordered words."""
+        if self._store_values is None:
+            return None
+        return self.indices_cutlass() if self._CUTLASS_METADATA else self._canonical_pair()[1]
 
     def __tensor_flatten__(self):
         return ["_store_values", "_store_meta"], (self.original_shape, self.transposed, self._store_shape, self._store_layout)
@@ -432,22 +464,19 @@ class SparseSemiStructuredTensor(torch.Tensor):
                                         m, k, out.data_ptr(), N.stream_ptr()))
         return out
 
+    def indices_canonical(self):
+        """Metadata as the canonical nibble stream, whatever `_CUTLASS_METADATA` says."""
+        return self._canonical_pair()[1]
+
     def indices_cutlass(self):
         """Metadata in the CUTLASS-reordered layout the reference's `indices()` returns
-        (reorder_meta + ColumnMajorInterleaved<2>; csrc .cu:826-851)."""
-        meta = self.meta_tensor_cutlass.contiguous()
-        m, ncols = meta.shape
-        group, inter = (32, 4) if meta.dtype == torch.int16 else (16, 2)
-        r = torch.arange(m, device=meta.device).view(-1, 1).expand(m, ncols)
-        c = torch.arange(ncols, device=meta.device).view(1, -1).expand(m, ncols)
-        dr = r // group * group + (r % 8) * inter + (r % group) // 8
-        tr = ((dr % 2 == 0) & (c % 2 == 1)).long()
-        bl = ((dr % 2 == 1) & (c % 2 == 0)).long()
-        dr, dc = dr + tr - bl, c - tr + bl
-        dest = (dc // 2) * m * 2 + dr * 2 + dc % 2
-        out = torch.empty_like(meta).view(-1)
-        out[dest.reshape(-1)] = meta.reshape(-1)
-        return out.view(m, ncols)
+        (reorder_meta + ColumnMajorInterleaved<2>; csrc .cu:826-851; semi_structured.py:536-546)."""
+        if self._store_layout == N.COMPRESSED_CUTLASS:
+            m, _ = self._store_shape
+            return self._store_meta.view(m, -1)
+        if self._cutlass is None:
+            self._cutlass = self._converted_meta(N.COMPRESSED_CUTLASS)
+        return self._cutlass
 
 
 def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = False, MVUE24: bool = False,

@@ -75,8 +75,18 @@ typedef enum { TF24_ACT_NONE = 0, TF24_ACT_RELU = 1, TF24_ACT_SILU = 2, TF24_ACT
  *              A 256-row tile of one stage is then one contiguous 16 KB run of values and 2 (4) contiguous
  *              1 KB runs of metadata, all copied to LDS with full-line GLOBAL_LOAD_LDS_DWORDX4, and the
  *              metadata lands in the order the matrix instructions' index operands are read in.
+ *   CUTLASS    the form the reference stores and hands to its matmul binding: values as CANONICAL, metadata
+ *              words (int16 for 16-bit values, int32 for 8-bit ones) permuted by CUTLASS's reorder_meta and
+ *              stored ColumnMajorInterleaved<2> (sparse/csrc/mySparseSemiStructuredLinear_cuda.cu:826-851; the
+ *              gather form of sparse/_semi_structured_conversions.py:178-213): canonical word (r, c) of the
+ *              [m, k/16 | k/32] word matrix goes to row r/G*G + (r%8)*I + (r%G)/8 with (G, I) = (32, 4) for
+ *              int16 and (16, 2) for int32 words, is swapped inside 2 x 2 blocks (even row, odd column <->
+ *              odd row, even column), and lands at word (c'/2)*2m + 2r' + c'%2.  This is what
+ *              SparseSemiStructuredTensor.indices() returns in the reference (sparse/semi_structured.py:536-546).
+ *              Accepted as an input of tf24_repack_to, tf24_decompress and tf24_spmm (which then runs its
+ *              general kernel: repack once to PANEL for speed) and produced by tf24_repack_to.
  */
-typedef enum { TF24_COMPRESSED_CANONICAL = 0, TF24_COMPRESSED_PANEL = 1 } tf24_compressed_layout;
+typedef enum { TF24_COMPRESSED_CANONICAL = 0, TF24_COMPRESSED_PANEL = 1, TF24_COMPRESSED_CUTLASS = 2 } tf24_compressed_layout;
 
 /* Library version string, e.g. "tf24 0.1.0 gfx950". Host only. */
 const char* tf24_version(void);
@@ -189,8 +199,9 @@ int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld, int64_t m
 /*
  * Compressed -> dense.  Replaces _sparse_semi_structured_to_dense_kernel
  * (sparse/_semi_structured_conversions.py:1163-1274) used by SparseSemiStructuredTensor.to_dense
- * (sparse/semi_structured.py:554-572).  values / meta in `layout`, dense_out [m,k] row-major
- * contiguous of the same dtype.
+ * (sparse/semi_structured.py:554-572).  values / meta in `layout` (any of the three; CUTLASS is the form
+ * the reference's own decompression starts from, :217-290), dense_out [m,k] row-major contiguous of the
+ * same dtype.
  */
 int tf24_decompress(const void* values, int dtype, const void* meta, int layout, int64_t m, int64_t k,
                     void* dense_out, void* stream);
@@ -205,6 +216,19 @@ int tf24_decompress(const void* values, int dtype, const void* meta, int layout,
  */
 int tf24_repack(const void* values_in, const void* meta_in, int dtype, int64_t m, int64_t k, int from_layout,
                 void* values_out, void* meta_out, void* stream);
+
+/*
+ * Storage conversion between any two of CANONICAL, PANEL and CUTLASS (out of place, from_layout != to_layout).
+ * With from_layout CUTLASS this is the import of a compressed operand as the reference stores it -- the
+ * (weight, meta) pair its matmul binding takes (sparse/sparse_semi_structured_linear.py:4-5) and
+ * SparseSemiStructuredTensor.values() / indices() return (sparse/semi_structured.py:526-546); with to_layout
+ * CUTLASS it is the reference's reordering step itself (sparse/_semi_structured_conversions.py:178-213,
+ * Triton :639-661 and :1047-1069).  m % 32 == 0; k % 64 == 0 (16-bit values) / k % 128 == 0 (8-bit).
+ * values_out may be NULL when neither side is PANEL (the values of CANONICAL and CUTLASS are the same bytes):
+ * then only the metadata is converted.
+ */
+int tf24_repack_to(const void* values_in, const void* meta_in, int dtype, int64_t m, int64_t k, int from_layout,
+                   int to_layout, void* values_out, void* meta_out, void* stream);
 
 /*
  * Transposable 4x4 mask search over the 90 row-and-column 2:4 patterns.
@@ -282,7 +306,8 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * Replaces sparse.cutlass.my_sparse_semi_structured_linear
  * (sparse/csrc/mySparseSemiStructuredLinear_cuda.cu:498-817, CUTLASS SparseGemm :61-76),
  * bound at sparse/sparse_semi_structured_linear.py:4-5.
- *   a_values, a_meta  the compressed operand in a_layout; dtype F16|BF16|E4M3|E5M2|I8 (B has the same dtype).
+ *   a_values, a_meta  the compressed operand in a_layout (PANEL: the fast kernels; CANONICAL and CUTLASS -- the
+ *              reference's own storage, .cu:826-851 -- run the general kernel); dtype F16|BF16|E4M3|E5M2|I8 (B has the same dtype).
  *              I8 is the integer product of .cu:594-637: int32 accumulation, out_dtype and bias I32,
  *              activation none or ReLU, scale 1; every other dtype accumulates in float32 and takes
  *              out_dtype F16|BF16|F32 with a bias of that type
@@ -301,7 +326,7 @@ int tf24_masked_add(void* grad, int grad_dtype, const void* p, int p_dtype, cons
  * n_dense % 8 == 0 (16-bit) / 16 (8-bit).  Leading dimensions: ldb a multiple of 8 (16-bit) / 16 (8-bit)
  * elements and at most 16 MiB per row (a tile's rows are addressed by 32-bit offsets), ldc a multiple of 8 for
  * 16-bit outputs and of 4 for 32-bit ones (16-byte row segments); b, c, a_values 16-byte aligned, a_meta 16-byte
- * aligned in panel form (8 in canonical form).
+ * aligned in panel form (8 in canonical form, 4 in CUTLASS form).
  */
 int tf24_spmm(const void* a_values, const void* a_meta, int a_layout, int dtype, int64_t n_sparse, int64_t k,
               const void* b, int b_layout, int64_t ldb, int64_t n_dense,

@@ -35,28 +35,42 @@ def test_forwarder_takes_the_reference_keywords(cuda):
         fn(x, values, meta, activation_opt="tanh")
 
 
-def test_forwarder_keeps_the_panel_copy_of_canonical_operands(cuda):
-    """Canonical (values, meta) tensors are repacked once, not per call; an in-place update of the
-    values is seen."""
-    import sys
+def test_forwarder_sees_every_rewrite_of_raw_operands(cuda):
+    """Raw (values, meta) tensors are repacked on every call: a rewrite that no version counter records
+    (`.data`, a kernel writing through the raw pointer) must change the product; inference-mode tensors
+    (which have no version counter) are accepted; a wrapper keeps its own panel copy."""
     import sparse
-    mod = sys.modules["sparse.sparse_semi_structured_linear"]     # the module; the package attribute of that name is the function
+    from sparse import _native as N
     w = _small_ints((128, 256), 4).half()
     x = _small_ints((64, 256), 5).half().to(cuda)
     mask = oracle.prune24_mask(w.float())
     ref = oracle.spmm_ref(x.float().cpu(), torch.where(mask, w.float(), torch.zeros(())))
     s = sparse.to_sparse_semi_structured(w.to(cuda))
     values, meta = s.values().clone(), s.indices().clone()
-    mod._PANEL_CACHE.clear()
-    assert sparse.sparse_semi_structured_linear(x, values, meta).float().cpu().equal(ref)
-    assert len(mod._PANEL_CACHE) == 1
-    wrapper = next(iter(mod._PANEL_CACHE.values()))[1]
-    panel_ptr = wrapper._store_values.data_ptr()
-    assert sparse.sparse_semi_structured_linear(x, values, meta).float().cpu().equal(ref)
-    assert next(iter(mod._PANEL_CACHE.values()))[1] is wrapper and wrapper._store_values.data_ptr() == panel_ptr
-    values.mul_(2)                                                   # in place: version counter moves, entry is rebuilt
-    assert sparse.sparse_semi_structured_linear(x, values, meta).float().cpu().equal(2 * ref)
-    mod._PANEL_CACHE.clear()
+    fn = sparse.sparse_semi_structured_linear
+    assert fn(x, values, meta).float().cpu().equal(ref)
+    version = values._version
+    values.data.mul_(2)                                              # does not move the version counter
+    assert values._version == version
+    assert fn(x, values, meta).float().cpu().equal(2 * ref)
+    # rewritten through the C ABI: the library's own kernels write through raw pointers
+    w2 = _small_ints((128, 256), 6).half()
+    mask2 = oracle.prune24_mask(w2.float())
+    ref2 = oracle.spmm_ref(x.float().cpu(), torch.where(mask2, w2.float(), torch.zeros(())))
+    w2g = w2.to(cuda)
+    N.check(N.lib().tf24_prune_compress(w2g.data_ptr(), N.F16, N.ROW_MAJOR, 256, 128, 256, N.PRUNE_MAGNITUDE, None, N.U8, 0, None, 0,
+                                        values.data_ptr(), N.F16, meta.data_ptr(), N.COMPRESSED_CANONICAL, N.stream_ptr()))
+    assert fn(x, values, meta).float().cpu().equal(ref2)
+    with torch.inference_mode():
+        vi, mi = values.clone(), meta.clone()
+        assert fn(x, vi, mi).float().cpu().equal(ref2)
+    # a wrapper owns its storage: the panel copy made by the first product is kept
+    wrapper = sparse.SparseSemiStructuredTensor(None, original_shape=torch.Size([128, 256]), sparse_tensor_cutlass=values,
+                                                meta_tensor_cutlass=meta, dtype=torch.float16)
+    assert fn(x, wrapper).float().cpu().equal(ref2)
+    assert wrapper._store_layout == N.COMPRESSED_PANEL
+    kept = wrapper._store_values.data_ptr()
+    assert fn(x, wrapper).float().cpu().equal(ref2) and wrapper._store_values.data_ptr() == kept
 
 
 @pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.int8, torch.float16])
@@ -125,3 +139,100 @@ def test_torch_named_operators(cuda):
     flat = torch.randn(24, generator=g)                                      # one dimension, 8 | numel
     sp, mask = sparse.sparse24_torch(flat.to(cuda))
     assert sp.cpu().equal(oracle.sparse24_dense(flat.view(-1, 8))[0].view(-1)) and mask.sum().item() == 12
+
+
+@pytest.mark.parametrize("dtype,m,k", [(torch.float16, 64, 256), (torch.bfloat16, 352, 704), (torch.float8_e4m3fn, 96, 640),
+                                       (torch.int8, 32, 128), (torch.float16, 32, 64)])
+def test_repack_to_and_from_the_reference_storage(cuda, dtype, m, k):
+    """tf24_repack_to between the canonical, panel and CUTLASS-reordered forms (int16 and int32 metadata
+    words), against the oracle's reorder (pinned by upstream PyTorch's converter); tf24_decompress from the
+    reordered form."""
+    import sparse
+    from sparse import _native as N
+    if dtype == torch.int8:
+        w = _small_ints((m, k), 11, -20, 21).to(torch.int8)
+    else:
+        w = _small_ints((m, k), 11).bfloat16()
+    want_v, want_m = oracle.compress24(w, out_dtype=dtype)
+    want_r = oracle.cutlass_reorder_meta(want_m)
+    s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=dtype)
+    code = N.operand_code(dtype)
+    pv, pm = s._store_values.contiguous(), s._store_meta.contiguous()
+    cv, cm = s.values().contiguous(), s.indices().contiguous()
+    lib = N.lib()
+
+    def repack(vin, min_, frm, to, with_values=True):
+        ov, om = torch.empty_like(pv), torch.empty_like(pm)
+        N.check(lib.tf24_repack_to(vin.data_ptr() if with_values else None, min_.data_ptr(), code, m, k, frm, to,
+                                   ov.data_ptr() if with_values else None, om.data_ptr(), N.stream_ptr()))
+        return ov, om
+
+    def same(t, want):
+        return t.view(torch.uint8).cpu().reshape(-1).equal(want.contiguous().view(torch.uint8).reshape(-1))
+
+    rv, rm = repack(cv, cm, N.COMPRESSED_CANONICAL, N.COMPRESSED_CUTLASS)          # the reference's reordering step
+    assert same(rv, want_v) and same(rm, want_r)
+    _, rm2 = repack(cv, cm, N.COMPRESSED_CANONICAL, N.COMPRESSED_CUTLASS, with_values=False)
+    assert same(rm2, want_r)
+    rv3, rm3 = repack(pv, pm, N.COMPRESSED_PANEL, N.COMPRESSED_CUTLASS)
+    assert same(rv3, want_v) and same(rm3, want_r)
+    bv, bm = repack(rv, rm, N.COMPRESSED_CUTLASS, N.COMPRESSED_CANONICAL)          # import: back to the nibble stream
+    assert same(bv, want_v) and same(bm, want_m)
+    qv, qm = repack(rv, rm, N.COMPRESSED_CUTLASS, N.COMPRESSED_PANEL)              # import: straight to the matmul's form
+    assert same(qv, pv.cpu()) and same(qm, pm.cpu())
+    dense = torch.empty((m, k), dtype=dtype, device=cuda)
+    N.check(lib.tf24_decompress(rv.data_ptr(), code, rm.data_ptr(), N.COMPRESSED_CUTLASS, m, k, dense.data_ptr(), N.stream_ptr()))
+    assert same(dense, oracle.decompress24(want_v, want_m))
+    with pytest.raises(RuntimeError):
+        N.check(lib.tf24_repack_to(cv.data_ptr(), cm.data_ptr(), code, m, k, N.COMPRESSED_CUTLASS, N.COMPRESSED_CUTLASS,
+                                   rv.data_ptr(), rm.data_ptr(), N.stream_ptr()))
+    with pytest.raises(RuntimeError):
+        N.check(lib.tf24_repack_to(cv.data_ptr(), cm.data_ptr(), code, m, k + 8, N.COMPRESSED_CANONICAL, N.COMPRESSED_CUTLASS,
+                                   rv.data_ptr(), rm.data_ptr(), N.stream_ptr()))
+
+
+@pytest.mark.parametrize("dtype,n,k,j", [(torch.float16, 32, 128, 24), (torch.float16, 352, 640, 296), (torch.bfloat16, 4128, 256, 520),
+                                         (torch.float8_e4m3fn, 352, 640, 304), (torch.int8, 96, 256, 48)])
+def test_product_from_reference_ordered_metadata(cuda, dtype, n, k, j):
+    """x . W^T with W given the way the reference's binding takes it (sparse_semi_structured_linear.py:4-5): row-major
+    values + CUTLASS-reordered metadata made by the oracle, never seen by this library's compression.  Through
+    the functional entry point (`meta_layout`), through the C ABI directly (the general kernel reads the
+    reordered words) and through a wrapper built with the class flag; exact on small integers."""
+    import sparse
+    from sparse import _native as N
+    lo, hi = (-20, 21) if dtype == torch.int8 else (-3, 4)
+    w = _small_ints((n, k), 21, lo, hi).to(dtype)
+    x = _small_ints((j, k), 22, -2, 3).to(dtype)
+    mask = oracle.prune24_mask(w.float())
+    ref = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(())))
+    values, meta = oracle.compress24(w.float(), out_dtype=dtype) if dtype != torch.int8 else oracle.compress24(w, out_dtype=dtype)
+    reordered = oracle.cutlass_reorder_meta(meta)
+    vg, mg, xg = values.to(cuda), reordered.to(cuda), x.to(cuda)
+    odt = torch.int32 if dtype == torch.int8 else torch.float32 if dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else dtype
+    want = ref.to(odt).float()
+    out = sparse.sparse_semi_structured_linear(xg, vg, mg, meta_layout="cutlass")
+    assert out.dtype == odt and out.float().cpu().equal(want)
+    if not reordered.equal(meta):
+        assert not sparse.sparse_semi_structured_linear(xg, vg, mg, meta_layout="canonical").float().cpu().equal(want)
+    # the C ABI on the reference's storage as it is
+    c = torch.empty((j, n), dtype=odt, device=cuda)
+    N.check(N.lib().tf24_spmm(vg.data_ptr(), mg.data_ptr(), N.COMPRESSED_CUTLASS, N.operand_code(dtype), n, k,
+                              xg.data_ptr(), N.ROW_MAJOR, k, j, c.data_ptr(), N.operand_code(odt), N.COL_MAJOR, n,
+                              None, 1.0, N.ACT_NONE, None, 0, N.stream_ptr()))
+    assert c.float().cpu().equal(want)
+    # the reference's tensor contract: constructor argument and indices() speak the reordered form
+    cls = sparse.SparseSemiStructuredTensor
+    cls._CUTLASS_METADATA = True
+    try:
+        s = cls(None, original_shape=torch.Size([n, k]), sparse_tensor_cutlass=vg, meta_tensor_cutlass=mg, dtype=dtype)
+        assert s.indices().cpu().equal(reordered) and s.meta_tensor_cutlass.cpu().equal(reordered)
+        assert s.indices_canonical().cpu().equal(meta)
+        assert s.values().cpu().view(torch.uint8).equal(values.view(torch.uint8))
+        assert torch.mm(xg, s.t()).float().cpu().equal(want)
+        assert s.to_dense().cpu().view(torch.uint8).equal(oracle.decompress24(values, meta).view(torch.uint8))
+        fresh = sparse.to_sparse_semi_structured(w.to(cuda) if dtype == torch.int8 else w.float().to(cuda), dtype=dtype)
+        assert fresh.indices().cpu().equal(reordered) and fresh.indices_cutlass().cpu().equal(reordered)
+        assert sparse.sparse_semi_structured_linear(xg, fresh.values(), fresh.indices()).float().cpu().equal(want)
+    finally:
+        cls._CUTLASS_METADATA = False
+    assert fresh.indices().cpu().equal(meta)

@@ -168,6 +168,32 @@ def test_config3_spmm_random_and_linear(cuda):
     assert float(normal.float().mean()) > 0.99
 
 
+def test_config3_spmm_bf16(cuda):
+    """bfloat16 at the size of config 3, both products: exact on small integers (sums stay below 2^24, one
+    rounding to bf16) and within 1e-2 of the float32 product on the config's random data."""
+    import sparse
+    g = torch.Generator(device=cuda).manual_seed(3)
+    x = torch.randint(-3, 4, (8192, 4096), device=cuda, generator=g).to(BF16)
+    w = torch.randint(-3, 4, (11008, 4096), device=cuda, generator=g).to(BF16)
+    dy = torch.randint(-3, 4, (8192, 11008), device=cuda, generator=g).to(BF16)
+    ws = sparse.to_sparse_semi_structured(w, dtype=BF16)
+    y = torch.mm(x, ws.t())
+    want = torch.mm(x.float(), ws.to_dense().float().t()).to(BF16)
+    assert y.dtype == BF16 and torch.equal(y.view(torch.int16), want.view(torch.int16))
+    _, tmask = sparse.TransposableSparse()(w)
+    wt = sparse.to_sparse_semi_structured(w.t(), mask=tmask.t(), dtype=BF16)
+    dx = torch.mm(dy, wt.t())
+    want = torch.mm(dy.float(), torch.where(tmask, w, torch.zeros_like(w)).float()).to(BF16)
+    assert torch.equal(dx.view(torch.int16), want.view(torch.int16))
+    del x, w, dy, want, y, dx
+    x = torch.randn(8192, 4096, device=cuda, generator=g).to(BF16)
+    w = (0.02 * torch.randn(11008, 4096, device=cuda, generator=g)).to(BF16)
+    ws = sparse.to_sparse_semi_structured(w, dtype=BF16)
+    y = torch.mm(x, ws.t())
+    ref = torch.mm(x.float(), ws.to_dense().float().t())
+    assert ((y.float() - ref).norm() / ref.norm()).item() < 1e-2
+
+
 def test_config5_fp8_spmm_rows_against_float32(cuda):
     import sparse
     g = torch.Generator(device=cuda).manual_seed(5)

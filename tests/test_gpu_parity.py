@@ -609,6 +609,38 @@ def test_spmm_chained_tiles_with_partial_edges(cuda, dtype, k):
     assert again.equal(out)
 
 
+@pytest.mark.parametrize("dtype,k,act,scale", [(F16, 256, "relu", 0.5), (BF16, 320, "relu", 1.0), (E4M3, 512, "relu", 0.25),
+                                               (F16, 320, "silu", 0.5), (BF16, 256, "gelu", 1.0), (E4M3, 640, "gelu", 0.125),
+                                               (F16, 256, "gelu", 1.0), (E5M2, 512, "silu", 1.0)])
+def test_spmm_chained_tiles_activation_and_scale(cuda, dtype, k, act, scale):
+    """The chained-tile kernel's third output pass (bias, scale and activation decided at run time): 17 x 17
+    tiles of 256 x 256 with partial edge tiles, more tiles than compute units.  Scale and bias act on exact
+    float32 sums of small integers, so ReLU results are exact (one rounding of an exact value); SiLU and
+    GELU are compared with torch's float32 functions of the same exact argument within 2e-3 + one unit in
+    the last place of the 16-bit output (the kernel's exp / erf differ from torch's by a few float32 ulps)."""
+    import sparse
+    n, m = 4128, 4112
+    odt = torch.bfloat16 if dtype in FLOAT8 else dtype
+    w = _small_ints((n, k), 74, -2, 3).to(dtype)
+    x = _small_ints((m, k), 75, -2, 3).to(dtype)
+    bias = (_small_ints((n,), 76) * 0.5).to(odt)
+    mask = oracle.prune24_mask(w.float())
+    pre = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(()))) * scale + bias.float()
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    out = sparse.sparse_semi_structured_linear(x.to(cuda), s, bias_opt=bias.to(cuda), activation_opt=act, out_dtype=odt, scale=scale)
+    assert out.shape == (m, n) and out.dtype == odt
+    got = out.float().cpu()
+    if act == "relu":
+        assert got.equal(pre.clamp_min(0).to(odt).float())
+    else:
+        want = torch.nn.functional.silu(pre) if act == "silu" else torch.nn.functional.gelu(pre)
+        ulp = 2.0 ** -8 if odt == torch.bfloat16 else 2.0 ** -11
+        err = (got - want).abs()
+        assert bool((err <= 2e-3 + (2e-3 + ulp) * want.abs()).all()), float(err.max())
+    again = sparse.sparse_semi_structured_linear(x.to(cuda), s, bias_opt=bias.to(cuda), activation_opt=act, out_dtype=odt, scale=scale)
+    assert again.equal(out)
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16, E4M3, E5M2])
 def test_spmm_tiled_all_operand_positions(cuda, dtype):
     """Shapes large enough for the tiled kernel, with partial tiles: both operand positions, both
@@ -921,3 +953,40 @@ def test_spmm_narrow_one_wave_per_block(cuda, dtype, n, panels):
     out = sparse.sparse_semi_structured_linear(x.to(cuda)[:8], s, bias=bias.to(cuda), activation="relu")
     want = (ref[:8] + bias.float()).clamp_min(0)
     assert out.float().cpu().equal(want.to(out.dtype).float())
+
+
+def test_narrowing_edge_values(cuda):
+    """Float32 -> e4m3 / e5m2 / bf16 / f16 on the device (hardware conversions where gfx950 has them) against
+    torch's casts, byte for byte, on the values where narrowing rules differ between implementations:
+    the largest finite value and the first one past it (e4m3: 448, ties at 464, NaN from 480 on -- not
+    saturation), e5m2's 57344 / 61440 and overflow to infinity, signed infinities and NaNs, signed zeros,
+    the subnormal boundaries and halfway cases of each type."""
+    import sparse
+    edge = [448.0, 449.0, 456.0, 463.99, 464.0, 464.01, 472.0, 479.9, 480.0, 512.0, 1e6, 57344.0, 59000.0, 61439.0, 61440.0, 61441.0,
+            65503.0, 65504.0, 65519.9, 65520.0, 65536.0, 1e30, float("inf"), float("nan"), 0.0,
+            2.0 ** -6, 2.0 ** -7, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -10, 2.0 ** -10 * 1.0001, 2.0 ** -11, 2.0 ** -14, 2.0 ** -16,
+            2.0 ** -17, 1.5 * 2.0 ** -17, 2.0 ** -18, 2.0 ** -24, 2.0 ** -25, 1.5 * 2.0 ** -25, 2.0 ** -126, 2.0 ** -133, 2.0 ** -149,
+            1.0, 1.0625, 1.09375, 1.125, 1.1875, 3.3895e38, 3.4e38, 240.0, 248.0, 0.0146484375, 0.015625]
+    vals = torch.tensor(edge + [-v for v in edge], dtype=torch.float32)
+    vals = torch.cat([vals, torch.tensor([0x7fa00001, 0xffc00123 - (1 << 32)], dtype=torch.int32).view(torch.float32)])   # NaNs with payloads
+    n = vals.numel()
+    k = 128
+    rows = (n + 1) // 2 * 4 // k + 1
+    rows = (rows + 31) // 32 * 32
+    # every value sits at position 0 or 1 of a group whose mask keeps exactly those two positions
+    dense = torch.zeros(rows * k, dtype=torch.float32)
+    idx = torch.arange(n)
+    dense[(idx // 2) * 4 + idx % 2] = vals
+    dense = dense.view(rows, k)
+    mask = torch.zeros(rows, k, dtype=torch.bool)
+    mask.view(-1, 4)[:, :2] = True
+    for odt in (E4M3, E5M2, BF16, F16):
+        s = sparse.to_sparse_semi_structured(dense.to(cuda), mask=mask.to(cuda), dtype=odt)
+        got = s.values().cpu().reshape(-1)[:n]
+        want = vals.to(odt)
+        gb, wb = got.view(torch.uint8 if odt in FLOAT8 else torch.int16), want.view(torch.uint8 if odt in FLOAT8 else torch.int16)
+        nan = vals != vals
+        assert gb[~nan].equal(wb[~nan]), (odt, vals[~nan][gb[~nan] != wb[~nan]])
+        assert bool((got[nan].float() != got[nan].float()).all()), odt          # NaN stays NaN (payloads are not compared for 16-bit types)
+        if odt in FLOAT8:
+            assert gb[nan].equal(wb[nan]), odt                                   # one NaN byte per sign, as torch's
