@@ -16,13 +16,12 @@ __device__ __forceinline__ uint32_t group_op(const float (&x)[4], float r0, floa
     // only the two kept values are rescaled; with fewer than two mask bits the kept element is
     // still one of the two encoded positions
     const Mvue4 g = mvue4(x[0], x[1], x[2], x[3], r0, r1);
-    const uint32_t nib = encode_nibble(g.mask);
-    const uint32_t pa = nib & 3, pb = nib >> 2;
-    const float ya = mvue_rescale(select4(pa, x[0], x[1], x[2], x[3]), select4(pa, g.p[0], g.p[1], g.p[2], g.p[3]), g.in_range);
-    const float yb = mvue_rescale(select4(pb, x[0], x[1], x[2], x[3]), select4(pb, g.p[0], g.p[1], g.p[2], g.p[3]), g.in_range);
+    const uint32_t pa = g.keep.nibble() & 3;
+    const float ya = mvue_rescale(g.keep.first(x[0], x[1], x[2]), g.keep.first(g.p[0], g.p[1], g.p[2]), g.in_range);
+    const float yb = mvue_rescale(g.keep.second(x[1], x[2], x[3]), g.keep.second(g.p[1], g.p[2], g.p[3]), g.in_range);
 #pragma unroll
     for (int i = 0; i < 4; i++) y[i] = (uint32_t)i == pa ? ya : yb;
-    return g.mask;
+    return g.keep.bits();
   } else {
     uint32_t mb = magnitude_mask4(x[0], x[1], x[2], x[3]);
     if constexpr (OP == OP_SOFT) {

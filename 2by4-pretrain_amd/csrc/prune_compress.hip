@@ -21,29 +21,49 @@ constexpr int kThreads = 256;
 // uniforms) one unit per lane and four times the blocks is (MVUE24 82 against 85 us, mask 67 against 71).
 template <int MODE> constexpr int unroll_for() { return MODE == TF24_PRUNE_MAGNITUDE ? 4 : 1; }
 
-// Kept-mask bits of one group; in MVUE mode also the inclusion probabilities the two kept
+// The kept elements of one group; in MVUE mode also the inclusion probabilities the two kept
 // values are divided by.
 template <typename In, int MODE, typename MaskT>
-__device__ __forceinline__ uint32_t prune_group(const float (&x)[4], const MaskT* mk, float r0, float r1, Mvue4& g) {
+__device__ __forceinline__ Keep4 prune_group(const float (&x)[4], const MaskT* mk, float r0, float r1, Mvue4& g) {
   if constexpr (MODE == TF24_PRUNE_MAGNITUDE) {
-    return magnitude_mask4(x[0], x[1], x[2], x[3]);
+    return magnitude_keep4(x[0], x[1], x[2], x[3]);
   } else if constexpr (MODE == TF24_PRUNE_MASK) {
-    uint32_t b = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) b |= (uint32_t)(to_float(mk[i]) != 0.0f) << i;
-    return b;
+    return Keep4{to_float(mk[0]) != 0.0f, to_float(mk[1]) != 0.0f, to_float(mk[2]) != 0.0f, to_float(mk[3]) != 0.0f};
   } else {
     g = mvue4(x[0], x[1], x[2], x[3], r0, r1);
-    return g.mask;
+    return g.keep;
   }
 }
 
-// The value stored for metadata position pos (0..3) of a group.
+// The two values stored for a group: the kept elements in ascending position (MVUE: rescaled).
 template <int MODE>
-__device__ __forceinline__ float kept_value(uint32_t pos, const float (&x)[4], const Mvue4& g) {
-  float v = select4(pos, x[0], x[1], x[2], x[3]);
-  if constexpr (MODE == TF24_PRUNE_MVUE) v = mvue_rescale(v, select4(pos, g.p[0], g.p[1], g.p[2], g.p[3]), g.in_range);
-  return v;
+__device__ __forceinline__ void kept_values(const Keep4& keep, const float (&x)[4], const Mvue4& g, float& first, float& second) {
+  first = keep.first(x[0], x[1], x[2]);
+  second = keep.second(x[1], x[2], x[3]);
+  if constexpr (MODE == TF24_PRUNE_MVUE) {
+    first = mvue_rescale(first, keep.first(g.p[0], g.p[1], g.p[2]), g.in_range);
+    second = mvue_rescale(second, keep.second(g.p[1], g.p[2], g.p[3]), g.in_range);
+  }
+}
+
+// Panel output of the row-major kernels: the metadata words of a block ([k/32][m][4 bytes]: one word per
+// row and 32 dense columns) are collected in LDS as [block of 32 columns][row] and leave as 16-byte
+// pieces of four adjacent rows, whole runs of `rows` words per block of columns.  Stored by the quad
+// leaders directly they are 4-byte pieces in 16 places per wave instruction, and partial writes of that
+// size cost the memory system whole bursts (magnitude, bf16 -> fp16 at 8192 x 8192: 38.6 us; the same
+// kernel with canonical output, whose words are contiguous: 34.4).
+// words = rows * kblocks metadata words of the block (at most kThreads); rows % 4 == 0.
+__device__ __forceinline__ void store_panel_meta_block(const uint32_t* s_words, int rows, int kblocks, int64_t row0, int64_t mbyte0,
+                                                       int64_t upr, int64_t m, uint8_t* __restrict__ meta) {
+  const int t4 = threadIdx.x * 4;
+  if (t4 < rows * kblocks) {
+    const int kb = t4 / rows, r = t4 - kb * rows;
+    const int64_t mbyte = mbyte0 + (int64_t)kb * 4;
+    if (mbyte < upr) {
+      const uint4 w = *reinterpret_cast<const uint4*>(s_words + t4);
+      *reinterpret_cast<uint4*>(meta + panel_meta_offset(mbyte, row0 + r, m)) = w;
+    }
+  }
 }
 
 // ------------------------------------------------------------------ row-major
@@ -62,6 +82,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
                    Out* __restrict__ values, uint8_t* __restrict__ meta, bool contiguous, bool panel, int lpr_shift) {
   constexpr int kUnroll = unroll_for<MODE>();
   constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
+  __shared__ __attribute__((aligned(16))) uint32_t s_words[kUnroll * kThreads / 4];
   const int64_t upr = k >> 3;                             // 8-element units per row
   const int64_t total = m * upr;
   const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
@@ -120,11 +141,12 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
         Mvue4 pr;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = to_float(in.v[4 * g + i]);
-        uint32_t mb = prune_group<In, MODE, MaskT>(x, &mk.v[4 * g], r[2 * g], r[2 * g + 1], pr);
-        uint32_t nib = encode_nibble(mb);
-        out.v[2 * g] = from_float<Out>(kept_value<MODE>(nib & 3, x, pr));
-        out.v[2 * g + 1] = from_float<Out>(kept_value<MODE>(nib >> 2, x, pr));
-        mbyte |= nib << (4 * g);
+        const Keep4 keep = prune_group<In, MODE, MaskT>(x, &mk.v[4 * g], r[2 * g], r[2 * g + 1], pr);
+        float v0, v1;
+        kept_values<MODE>(keep, x, pr, v0, v1);
+        out.v[2 * g] = from_float<Out>(v0);
+        out.v[2 * g + 1] = from_float<Out>(v1);
+        mbyte |= keep.nibble() << (4 * g);
       }
       out.store_stream(values + ounit * 4);
     }
@@ -133,7 +155,18 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
     w |= __shfl_down(mbyte, 1) << 8;
     w |= __shfl_down(mbyte, 2) << 16;
     w |= __shfl_down(mbyte, 3) << 24;
-    if (live && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ometa) = w;
+    if (panel) {
+      const int rpi = kThreads >> lpr_shift;
+      if ((threadIdx.x & 3) == 0)
+        s_words[((threadIdx.x & ((1 << lpr_shift) - 1)) >> 2) * (kUnroll * rpi) + it * rpi + (threadIdx.x >> lpr_shift)] = w;
+    } else if (live && (threadIdx.x & 3) == 0) {
+      *reinterpret_cast<uint32_t*>(meta + ometa) = w;
+    }
+  }
+  if (panel) {
+    __syncthreads();
+    const int rows = kUnroll * (kThreads >> lpr_shift);
+    store_panel_meta_block(s_words, rows, 1 << (lpr_shift - 2), (int64_t)blockIdx.y * rows, (int64_t)blockIdx.x << lpr_shift, upr, m, meta);
   }
 }
 
@@ -150,6 +183,7 @@ prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, in
   constexpr int kUnroll = unroll_for<TF24_PRUNE_MAGNITUDE>();
   constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
   constexpr uint32_t kInf = std::is_same<In, f16_t>::value ? 0x7c00u : 0x7f80u;
+  __shared__ __attribute__((aligned(16))) uint32_t s_words[kUnroll * kThreads / 4];
   const int64_t upr = k >> 3;
   const int64_t total = m * upr;
   const int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
@@ -210,7 +244,18 @@ prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, in
     w |= __shfl_down(mbyte, 1) << 8;
     w |= __shfl_down(mbyte, 2) << 16;
     w |= __shfl_down(mbyte, 3) << 24;
-    if (live[it] && (threadIdx.x & 3) == 0) *reinterpret_cast<uint32_t*>(meta + ometa[it]) = w;
+    if (panel) {
+      const int rpi = kThreads >> lpr_shift;
+      if ((threadIdx.x & 3) == 0)
+        s_words[((threadIdx.x & ((1 << lpr_shift) - 1)) >> 2) * (kUnroll * rpi) + it * rpi + (threadIdx.x >> lpr_shift)] = w;
+    } else if (live[it] && (threadIdx.x & 3) == 0) {
+      *reinterpret_cast<uint32_t*>(meta + ometa[it]) = w;
+    }
+  }
+  if (panel) {
+    __syncthreads();
+    const int rows = kUnroll * (kThreads >> lpr_shift);
+    store_panel_meta_block(s_words, rows, 1 << (lpr_shift - 2), (int64_t)blockIdx.y * rows, (int64_t)blockIdx.x << lpr_shift, upr, m, meta);
   }
 }
 
@@ -292,11 +337,13 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       float u0 = 0.f, u1 = 0.f;
       if constexpr (MODE == TF24_PRUNE_MVUE) { u0 = rr[0].v[i]; u1 = rr[1].v[i]; }
       if (rowsum_partial) psum[i] = (x[0] + x[1]) + (x[2] + x[3]);
-      uint32_t mb = prune_group<In, MODE, MaskT>(x, mrow, u0, u1, pr);
-      uint32_t nib = encode_nibble(mb);
+      const Keep4 keep = prune_group<In, MODE, MaskT>(x, mrow, u0, u1, pr);
+      const uint32_t nib = keep.nibble();
+      float v0, v1;
+      kept_values<MODE>(keep, x, pr, v0, v1);
       Pack<Out, 2> o;
-      o.v[0] = from_float<Out>(kept_value<MODE>(nib & 3, x, pr));
-      o.v[1] = from_float<Out>(kept_value<MODE>(nib >> 2, x, pr));
+      o.v[0] = from_float<Out>(v0);
+      o.v[1] = from_float<Out>(v1);
       const int lr = rchunk * R + i;
       o.store(reinterpret_cast<Out*>(s_val + lr * VPITCH) + grp * 2);
       // two groups share a metadata byte: even group low nibble, odd group high nibble
@@ -396,6 +443,9 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
     const int lpr_shift = m % (kUnroll * (kThreads >> 4)) == 0 ? 4 : 5;
     if (panel) {
       const int rows_per_block = kUnroll * (kThreads >> lpr_shift), units_per_block = 1 << lpr_shift;
+      if (m / rows_per_block > 65535)
+        return fail(TF24_ERR_SHAPE, "tf24_prune_compress: %lld rows exceed the %lld the panel-output kernel of this mode covers in one launch; "
+                    "write the canonical layout and convert it with tf24_repack", (long long)m, (long long)65535 * rows_per_block);
       grid = dim3((unsigned)(((k >> 3) + units_per_block - 1) / units_per_block), (unsigned)(m / rows_per_block));
     }
     if constexpr (MODE == TF24_PRUNE_MAGNITUDE && (std::is_same<In, f16_t>::value || std::is_same<In, bf16_t>::value)) {
@@ -482,6 +532,8 @@ int run_prune_compress(const char* fn, const void* dense, int in_dtype, int layo
   if ((rc = check_aligned(fn, 8, {meta, mask}))) return rc;
   if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
     return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, out_layout);
+  // panel metadata leaves (and is later copied to LDS by the matmul) in 16-byte pieces
+  if (out_layout == TF24_COMPRESSED_PANEL && (rc = check_aligned(fn, 16, {meta}))) return rc;
   const bool panel = out_layout == TF24_COMPRESSED_PANEL;
   RandSrc rs{rnd, rand_ld, mode == TF24_PRUNE_MVUE_PACKED ? RAND_PACKED : RAND_FULL, 0, 0};
   if (mode == TF24_PRUNE_MVUE_SEEDED) {          // `rand` points to {seed, offset} in host memory

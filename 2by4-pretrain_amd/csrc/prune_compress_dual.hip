@@ -69,24 +69,24 @@ prune_compress_dual(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t
         ounit = panel ? ((col8 / UPP) * m + row) * UPP + col8 % UPP : row * upr + col8;
         ometa = panel ? panel_meta_offset(col8, row, m) : ounit;
         Out cv[8];
-        uint32_t keep = 0;
+        bool kept[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
           cv[i] = from_float<Out>(to_float(in.v[i]));
-          keep |= (uint32_t)(to_float(mk.v[i]) != 0.0f) << i;
+          kept[i] = to_float(mk.v[i]) != 0.0f;
         }
         Pack<Out, 4> out;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
-          const uint32_t nib = encode_nibble((keep >> (4 * g)) & 15u);
-          out.v[2 * g] = select4(nib & 3, cv[4 * g], cv[4 * g + 1], cv[4 * g + 2], cv[4 * g + 3]);
-          out.v[2 * g + 1] = select4(nib >> 2, cv[4 * g], cv[4 * g + 1], cv[4 * g + 2], cv[4 * g + 3]);
-          mbyte |= nib << (4 * g);
+          const Keep4 keep{kept[4 * g], kept[4 * g + 1], kept[4 * g + 2], kept[4 * g + 3]};
+          out.v[2 * g] = keep.first(cv[4 * g], cv[4 * g + 1], cv[4 * g + 2]);
+          out.v[2 * g + 1] = keep.second(cv[4 * g + 1], cv[4 * g + 2], cv[4 * g + 3]);
+          mbyte |= keep.nibble() << (4 * g);
         }
         out.store_stream(values + ounit * 4);
         Pack<E, 8> e;
 #pragma unroll
-        for (int i = 0; i < 8; i++) e.v[i] = (E)(bits_of(cv[i]) | (((keep >> i) & 1u) << KEEP));
+        for (int i = 0; i < 8; i++) e.v[i] = (E)(bits_of(cv[i]) | (kept[i] ? 1u << KEEP : 0u));
         e.store(tile + lr * TC + ((c8 * 8) ^ ((lr / RL) * SW)));
       }
       // 4 adjacent lanes (32 dense columns of one row) -> one metadata dword
@@ -115,11 +115,10 @@ prune_compress_dual(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t
         uint32_t e[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) e[i] = tile[(q * RL + 4 * g + i) * TC + cc];
-        const uint32_t keep = ((e[0] >> KEEP) & 1u) | (((e[1] >> KEEP) & 1u) << 1) | (((e[2] >> KEEP) & 1u) << 2) | (((e[3] >> KEEP) & 1u) << 3);
-        const uint32_t nib = encode_nibble(keep);
-        o.v[2 * g] = out_from_bits<Out>(select4(nib & 3, e[0], e[1], e[2], e[3]));
-        o.v[2 * g + 1] = out_from_bits<Out>(select4(nib >> 2, e[0], e[1], e[2], e[3]));
-        mbits |= nib << (4 * g);
+        const Keep4 keep{((e[0] >> KEEP) & 1u) != 0, ((e[1] >> KEEP) & 1u) != 0, ((e[2] >> KEEP) & 1u) != 0, ((e[3] >> KEEP) & 1u) != 0};
+        o.v[2 * g] = out_from_bits<Out>(keep.first(e[0], e[1], e[2]));
+        o.v[2 * g + 1] = out_from_bits<Out>(keep.second(e[1], e[2], e[3]));
+        mbits |= keep.nibble() << (4 * g);
       }
       // 16 bytes of kept values: byte offset gbyte of the canonical row; panel p = gbyte / 64 of row
       // trow lives at (p * k + trow) * 64

@@ -219,28 +219,48 @@ struct Pack {
 };
 
 // ---------------------------------------------------------------- 2:4 group math
-// Magnitude mask: bit i set = element i kept.  Six strict compares of |x|; ties keep the
-// larger index (all equal -> elements 2 and 3).
-__device__ __forceinline__ uint32_t magnitude_mask4(float x0, float x1, float x2, float x3) {
+// The kept elements of one group as four flags, and what the reference's 16-row table
+// (_semi_structured_conversions.py:46-82) makes of them: idx0 = 0 if m0, else 1 if m1, else 2;
+// idx1 = 1 if m0 & m1 & !m2, else 2 if m2 & (m0 | m1), else 3 -- for any of the 16 flag combinations, not
+// only the valid ones with two flags set.  Written on the flags themselves, which the compares leave
+// in scalar registers: picking a kept value is two selects on scalar conditions, where the route over
+// the packed nibble (bits -> positions -> compares -> three selects per value) costs three times the
+// vector instructions.
+struct Keep4 {
+  bool m0, m1, m2, m3;
+  __device__ __forceinline__ bool second_is_1() const { return m0 & m1 & !m2; }
+  __device__ __forceinline__ bool second_is_2() const { return m2 & (m0 | m1); }
+  template <typename T> __device__ __forceinline__ T first(T v0, T v1, T v2) const { return m0 ? v0 : (m1 ? v1 : v2); }
+  template <typename T> __device__ __forceinline__ T second(T v1, T v2, T v3) const { return second_is_1() ? v1 : (second_is_2() ? v2 : v3); }
+  // pos0 | pos1 << 2
+  __device__ __forceinline__ uint32_t nibble() const {
+    const uint32_t lo = m0 ? 0u : (m1 ? 1u : 2u);
+    const uint32_t hi = second_is_1() ? 4u : (second_is_2() ? 8u : 12u);
+    return lo | hi;
+  }
+  __device__ __forceinline__ uint32_t bits() const { return (uint32_t)m0 | ((uint32_t)m1 << 1) | ((uint32_t)m2 << 2) | ((uint32_t)m3 << 3); }
+};
+__device__ __forceinline__ Keep4 keep_from_bits(uint32_t mbits) { return Keep4{(mbits & 1) != 0, (mbits & 2) != 0, (mbits & 4) != 0, (mbits & 8) != 0}; }
+
+// Magnitude mask.  Six strict compares of |x|; ties keep the larger index (all equal -> elements 2 and 3).
+__device__ __forceinline__ Keep4 magnitude_keep4(float x0, float x1, float x2, float x3) {
   float a = __builtin_fabsf(x0), b = __builtin_fabsf(x1), c = __builtin_fabsf(x2), d = __builtin_fabsf(x3);
   bool x1_ = a > b, x2_ = a > c, x3_ = a > d, x4_ = b > c, x5_ = b > d, x6_ = c > d;
-  bool m0 = (x2_ & x3_) | (x1_ & x2_) | (x1_ & x3_);
-  bool m1 = (!x1_ & x5_) | (x4_ & x5_) | (!x1_ & x4_);
-  bool m2 = (!x2_ & !x4_) | (!x2_ & x6_) | (!x4_ & x6_);
-  bool m3 = (!x3_ & !x5_) | (!x3_ & !x6_) | (!x5_ & !x6_);
-  return (uint32_t)m0 | ((uint32_t)m1 << 1) | ((uint32_t)m2 << 2) | ((uint32_t)m3 << 3);
+  Keep4 k;
+  k.m0 = (x2_ & x3_) | (x1_ & x2_) | (x1_ & x3_);
+  k.m1 = (!x1_ & x5_) | (x4_ & x5_) | (!x1_ & x4_);
+  k.m2 = (!x2_ & !x4_) | (!x2_ & x6_) | (!x4_ & x6_);
+  k.m3 = (!x3_ & !x5_) | (!x3_ & !x6_) | (!x5_ & !x6_);
+  return k;
+}
+// the same as bits: bit i set = element i kept
+__device__ __forceinline__ uint32_t magnitude_mask4(float x0, float x1, float x2, float x3) {
+  return magnitude_keep4(x0, x1, x2, x3).bits();
 }
 
 // mask bits -> nibble pos0 | pos1<<2 (the 16-row table: masks with other than two bits set
 // are mapped as the reference's boolean minimisation maps them)
-__device__ __forceinline__ uint32_t encode_nibble(uint32_t mbits) {
-  bool m0 = mbits & 1, m1 = mbits & 2, m2 = mbits & 4;
-  bool bit0 = !m0 & m1;
-  bool bit1 = !m0 & !m1;
-  bool bit2 = bit1 | !m2;
-  bool bit3 = bit0 | !m1 | m2;
-  return (uint32_t)bit0 | ((uint32_t)bit1 << 1) | ((uint32_t)bit2 << 2) | ((uint32_t)bit3 << 3);
-}
+__device__ __forceinline__ uint32_t encode_nibble(uint32_t mbits) { return keep_from_bits(mbits).nibble(); }
 
 // Magnitude selection of one group of four 16-bit floats (f16 or bf16) held as two dwords
 // (x1:x0, x3:x2), in integer arithmetic: for numbers the order of |x| is the order of the low 15
@@ -330,7 +350,7 @@ struct RandSrc {
 // div_in_range; p_i >= t_i because k >= k_i for a rounded sum of non-negatives.
 struct Mvue4 {
   float p[4];
-  uint32_t mask;
+  Keep4 keep;
   bool in_range;
 };
 
@@ -341,7 +361,8 @@ __device__ __forceinline__ Mvue4 mvue4(float x0, float x1, float x2, float x3, f
   float sum = ((a0 + a1) + a2) + a3;
   float s0 = sum - a0, s1 = sum - a1, s2 = sum - a2, s3 = sum - a3;
   Mvue4 g;
-  g.in_range = (sum < 0x1p40f) & (s0 > 0.0f) & (s1 > 0.0f) & (s2 > 0.0f) & (s3 > 0.0f);
+  // every s_i > 0  <=>  their minimum is (none of them is a NaN when sum < 2^40: all a_i are finite then)
+  g.in_range = (sum < 0x1p40f) && (__builtin_fminf(__builtin_fminf(s0, s1), __builtin_fminf(s2, s3)) > 0.0f);
   float t0, t1, t2, t3, k0, k1, k2, k3;
   if (g.in_range) {
     const float rs = refined_rcp(sum);
@@ -367,7 +388,7 @@ __device__ __forceinline__ Mvue4 mvue4(float x0, float x1, float x2, float x3, f
   bool e1 = (t <= (d0 + d1)) & !e0;
   bool e2 = (t <= ((d0 + d1) + d2)) & !e1 & !e0;
   bool e3 = !e2 & !e1 & !e0;
-  g.mask = (uint32_t)(m0 | e0) | ((uint32_t)(m1 | e1) << 1) | ((uint32_t)(m2 | e2) << 2) | ((uint32_t)(m3 | e3) << 3);
+  g.keep.m0 = m0 | e0; g.keep.m1 = m1 | e1; g.keep.m2 = m2 | e2; g.keep.m3 = m3 | e3;
   return g;
 }
 
