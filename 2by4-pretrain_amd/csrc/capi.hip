@@ -65,7 +65,7 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
     return fail(TF24_ERR_DTYPE, "%s: unsupported output dtype %d", fn, out_dtype);
   if ((in_dtype == TF24_I8) != (out_dtype == TF24_I8))
     return fail(TF24_ERR_DTYPE, "%s: int8 values come from an int8 dense matrix only (input dtype %d, output dtype %d)", fn, in_dtype, out_dtype);
-  if (in_dtype == TF24_I8 && (mode == TF24_PRUNE_MVUE || mode == TF24_PRUNE_MVUE_PACKED || mode == TF24_PRUNE_MVUE_SEEDED))
+  if (in_dtype == TF24_I8 && (mode == TF24_PRUNE_MVUE || mode == TF24_PRUNE_MVUE_PACKED || mode == TF24_PRUNE_MVUE_SEEDED || mode == TF24_PRUNE_MVUE_SEEDED_DEVICE))
     return fail(TF24_ERR_ARG, "%s: MVUE24 rescales the kept values and is not defined for int8", fn);
   if (!is_layout(layout)) return fail(TF24_ERR_ARG, "%s: bad layout %d", fn, layout);
   const int64_t min_rows = 32, min_cols = is_8bit(out_dtype) ? 128 : 64;
@@ -98,6 +98,7 @@ extern "C" int tf24_prune_compress_validate(int in_dtype, int layout, int64_t ld
       if ((rc = check_ld(fn, "rand", layout, rand_ld, m, k / 2))) return rc;
       break;
     case TF24_PRUNE_MVUE_SEEDED:
+    case TF24_PRUNE_MVUE_SEEDED_DEVICE:
       if (!has_rand) return fail(TF24_ERR_ARG, "%s: mode MVUE_SEEDED needs `rand` to point to {seed, offset}", fn);
       break;
     default:

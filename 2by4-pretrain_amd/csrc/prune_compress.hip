@@ -121,7 +121,7 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
       if constexpr (MODE == TF24_PRUNE_MASK) mk.load_stream(mask + row * mask_ld + col8 * 8);
       if constexpr (MODE == TF24_PRUNE_MVUE) {
         if (rs.kind == RAND_SEEDED) {
-          const Philox4 c = philox4x32_10(rs.seed, (uint64_t)(row * upr + col8), rs.offset);
+          const Philox4 c = philox4x32_10(rs.seed_now(), (uint64_t)(row * upr + col8), rs.offset_now());
           r[0] = philox_uniform(c.x); r[1] = philox_uniform(c.y); r[2] = philox_uniform(c.z); r[3] = philox_uniform(c.w);
         } else if (rs.kind == RAND_PACKED) {                   // [m, k/2]: the unit's four uniforms are adjacent
           Pack<float, 4> r4;
@@ -299,7 +299,7 @@ prune_compress_col(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
 #pragma unroll
       for (int j = 0; j < R / 2; j++) {
         const int64_t row = r0 + j + par * (R / 2);
-        const Philox4 c = philox4x32_10(rs.seed, (uint64_t)(row * (k >> 3) + (c0 >> 3)), rs.offset);
+        const Philox4 c = philox4x32_10(rs.seed_now(), (uint64_t)(row * (k >> 3) + (c0 >> 3)), rs.offset_now());
         const float own0 = philox_uniform(par ? c.z : c.x), own1 = philox_uniform(par ? c.w : c.y);
         const float snd0 = philox_uniform(par ? c.x : c.z), snd1 = philox_uniform(par ? c.y : c.w);
         const float rcv0 = __shfl_xor(snd0, 8), rcv1 = __shfl_xor(snd1, 8);
@@ -429,6 +429,11 @@ rowsum_finish(const float* __restrict__ partial, int nblocks, int64_t m, T* __re
   }
 }
 
+// {seed, offset} in device memory: offset += by (vector store from one lane)
+__global__ void advance_philox_offset(uint64_t* state, uint64_t by) {
+  if (threadIdx.x == 0) state[1] += by;
+}
+
 template <typename In, typename Out, int MODE, typename MaskT>
 int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, const void* mask, int64_t mask_ld,
            RandSrc rs, void* values, void* meta, bool panel, float* rowsum_partial, hipStream_t stream) {
@@ -497,6 +502,7 @@ int dispatch_mode(int mode, const void* dense, int layout, int64_t ld, int64_t m
     case TF24_PRUNE_MVUE:
     case TF24_PRUNE_MVUE_PACKED:
     case TF24_PRUNE_MVUE_SEEDED:
+    case TF24_PRUNE_MVUE_SEEDED_DEVICE:
       if constexpr (std::is_same<Out, i8_t>::value) break;        // refused by the validator
       else return dispatch_mask<In, Out, TF24_PRUNE_MVUE>(dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
   }
@@ -528,26 +534,36 @@ int run_prune_compress(const char* fn, const void* dense, int in_dtype, int layo
                                         rnd != nullptr, rand_ld, out_dtype);
   if (rc != TF24_OK) return rc;
   if (!dense || !values || !meta) return fail(TF24_ERR_ARG, "%s: null dense/values/meta pointer", fn);
-  if ((rc = check_aligned(fn, 16, {dense, mode == TF24_PRUNE_MVUE_SEEDED ? nullptr : rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
+  if ((rc = check_aligned(fn, 16, {dense, (mode == TF24_PRUNE_MVUE_SEEDED || mode == TF24_PRUNE_MVUE_SEEDED_DEVICE) ? nullptr : rnd, values, mask_dtype == TF24_U8 ? nullptr : mask}))) return rc;
   if ((rc = check_aligned(fn, 8, {meta, mask}))) return rc;
   if (out_layout != TF24_COMPRESSED_CANONICAL && out_layout != TF24_COMPRESSED_PANEL)
     return fail(TF24_ERR_ARG, "%s: bad compressed layout %d", fn, out_layout);
   // panel metadata leaves (and is later copied to LDS by the matmul) in 16-byte pieces
   if (out_layout == TF24_COMPRESSED_PANEL && (rc = check_aligned(fn, 16, {meta}))) return rc;
   const bool panel = out_layout == TF24_COMPRESSED_PANEL;
-  RandSrc rs{rnd, rand_ld, mode == TF24_PRUNE_MVUE_PACKED ? RAND_PACKED : RAND_FULL, 0, 0};
+  RandSrc rs{rnd, rand_ld, mode == TF24_PRUNE_MVUE_PACKED ? RAND_PACKED : RAND_FULL, 0, 0, nullptr};
   if (mode == TF24_PRUNE_MVUE_SEEDED) {          // `rand` points to {seed, offset} in host memory
     const uint64_t* so = reinterpret_cast<const uint64_t*>(rnd);
-    rs = RandSrc{nullptr, 0, RAND_SEEDED, so[0], so[1]};
+    rs = RandSrc{nullptr, 0, RAND_SEEDED, so[0], so[1], nullptr};
+  } else if (mode == TF24_PRUNE_MVUE_SEEDED_DEVICE) {   // ... in device memory, read by the kernel
+    if ((rc = check_aligned(fn, 8, {rnd}))) return rc;
+    rs = RandSrc{nullptr, 0, RAND_SEEDED, 0, 0, reinterpret_cast<const uint64_t*>(rnd)};
   }
   hipStream_t s = (hipStream_t)stream;
+  rc = fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
   switch (in_dtype) {
-    case TF24_F32: return dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
-    case TF24_F16: return dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
-    case TF24_BF16: return dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
-    case TF24_I8: return dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s);
+    case TF24_F32: rc = dispatch_out<float>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s); break;
+    case TF24_F16: rc = dispatch_out<f16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s); break;
+    case TF24_BF16: rc = dispatch_out<bf16_t>(out_dtype, mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s); break;
+    case TF24_I8: rc = dispatch_mode<i8_t, i8_t>(mode, dense, layout, ld, m, k, mask, mask_dtype, mask_ld, rs, values, meta, panel, rowsum_partial, s); break;
   }
-  return fail(TF24_ERR_DTYPE, "%s: unsupported input dtype %d", fn, in_dtype);
+  if (rc == TF24_OK && mode == TF24_PRUNE_MVUE_SEEDED_DEVICE) {
+    // the generator state moves on behind the conversion, in stream order: the next sampling call (or the
+    // next replay of a graph holding this one) draws from a fresh offset
+    hipLaunchKernelGGL(advance_philox_offset, dim3(1), dim3(64), 0, s, const_cast<uint64_t*>(rs.state), (uint64_t)4);
+    rc = check_launch(fn);
+  }
+  return rc;
 }
 
 }  // namespace

@@ -339,6 +339,9 @@ struct RandSrc {
   int64_t ld;
   int kind;
   uint64_t seed, offset;  // RAND_SEEDED
+  const uint64_t* state;  // RAND_SEEDED: when not null, {seed, offset} are read from here (device memory) by the kernel
+  __device__ __forceinline__ uint64_t seed_now() const { return state ? state[0] : seed; }
+  __device__ __forceinline__ uint64_t offset_now() const { return state ? state[1] : offset; }
 };
 
 // MVUE24 of one group in float32, in the reference's operation order (no contraction): inclusion

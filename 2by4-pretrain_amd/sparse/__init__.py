@@ -5,8 +5,8 @@ every operator runs a hand-written HIP kernel from lib2by4_gfx950.so and raises 
 is missing -- there is no CPU or PyTorch fallback.
 """
 from .semi_structured import (SparseSemiStructuredTensor, to_sparse_semi_structured, to_sparse_semi_structured_pair,
-                              to_sparse_semi_structured_with_row_sums)
-from .transposable_semi_structured import TransposableSparse, mask_select
+                              to_sparse_semi_structured_with_row_sums, mvue_device_state)
+from .transposable_semi_structured import TransposableSparse, mask_select, transposable_mask_
 from .decay import masked_add_
 from .adamw import MaskedDecayAdamW
 from .adamw_step import AdamW_STEP
@@ -20,8 +20,8 @@ from .sparse_ops import MyLinear, SparseLinear, SoftThreshold, SoftThresholdLine
 
 __all__ = [
     "SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair",
-    "to_sparse_semi_structured_with_row_sums",
-    "TransposableSparse", "mask_select",
+    "to_sparse_semi_structured_with_row_sums", "mvue_device_state",
+    "TransposableSparse", "mask_select", "transposable_mask_",
     "masked_add_", "MaskedDecayAdamW", "AdamW_STEP",
     "soft_threshold24", "sparse24", "MVUE24_approx",
     "soft_threshold24_triton", "sparse24_triton", "MVUE24_approx_triton",

@@ -14,7 +14,7 @@ _lib = None
 # enums of tf24.h
 F32, F16, BF16, E4M3, U8, E5M2, I8, I32 = 0, 1, 2, 3, 4, 5, 6, 7
 ROW_MAJOR, COL_MAJOR = 0, 1
-PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE, PRUNE_MVUE_PACKED, PRUNE_MVUE_SEEDED = 0, 1, 2, 3, 4
+PRUNE_MAGNITUDE, PRUNE_MASK, PRUNE_MVUE, PRUNE_MVUE_PACKED, PRUNE_MVUE_SEEDED, PRUNE_MVUE_SEEDED_DEVICE = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_RELU, ACT_SILU, ACT_GELU = 0, 1, 2, 3
 COMPRESSED_CANONICAL, COMPRESSED_PANEL, COMPRESSED_CUTLASS = 0, 1, 2
 

@@ -27,7 +27,7 @@ import torch
 from . import _native as N
 
 __all__ = ["SparseSemiStructuredTensor", "to_sparse_semi_structured", "to_sparse_semi_structured_pair",
-           "to_sparse_semi_structured_with_row_sums"]
+           "to_sparse_semi_structured_with_row_sums", "mvue_device_state"]
 
 _Config = namedtuple("_SEMI_STRUCTURED_SPARSE_CONFIG",
                      "compression_factor sparse_min_rows sparse_min_cols dense_min_rows dense_min_cols")
@@ -75,10 +75,49 @@ class _HostWords:
         return ctypes.addressof(self.array)
 
 
+_DEVICE_PHILOX = {}        # device index -> int64[2] device tensor {seed, offset}
+
+
+def mvue_device_state(device=None, seed=None, offset=None):
+    """The {seed, offset} pair of MVUE24's in-kernel generator as a 2-element int64 tensor ON the device.
+
+    A sampling call that is given this tensor as `rand` reads the pair when its kernel runs and leaves
+    offset += 4 behind, in stream order -- so a HIP graph that holds MVUE24 conversions draws fresh,
+    reproducible uniforms on every replay (a (seed, offset) pair of host integers would be frozen into
+    the graph).  While a stream is being captured, MVUE24 conversions without an explicit `rand` use this
+    state; it has to exist before the capture starts: call this function first (it allocates and
+    copies).  `seed` / `offset` (re)initialise the state; by default it is created once from torch's
+    generator for the device (torch.manual_seed applies) and returned unchanged afterwards."""
+    if device is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    device = torch.device(device)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    state = _DEVICE_PHILOX.get(index)
+    if state is None or seed is not None or offset is not None:
+        gen = torch.cuda.default_generators[index]
+        s = gen.initial_seed() if seed is None else int(seed)
+        o = (gen.get_offset() if state is None else 0) if offset is None else int(offset)
+        signed = [v - (1 << 64) if v >= (1 << 63) else v for v in (s & (2 ** 64 - 1), o & (2 ** 64 - 1))]
+        words = torch.tensor(signed, dtype=torch.int64)
+        if state is None:
+            state = _DEVICE_PHILOX[index] = words.to(torch.device("cuda", index))
+        else:
+            state.copy_(words)
+    return state
+
+
 def _next_philox_state(device):
     """(seed, offset) of torch's generator for `device`, advancing its offset the way a random op does,
-    so that torch.manual_seed() makes the default MVUE24 sampling reproducible."""
-    gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+    so that torch.manual_seed() makes the default MVUE24 sampling reproducible.  Under stream capture:
+    the device-resident state of mvue_device_state()."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if torch.cuda.is_current_stream_capturing():
+        state = _DEVICE_PHILOX.get(index)
+        if state is None:
+            raise RuntimeError("MVUE24 under HIP graph capture takes its generator state from device memory: "
+                               "call sparse.mvue_device_state() once before the capture starts")
+        return state
+    gen = torch.cuda.default_generators[index]
     offset = gen.get_offset()
     gen.set_offset(offset + 4)
     return gen.initial_seed(), offset
@@ -119,7 +158,12 @@ def _compress(original, dtype, MVUE24, mask, rand, panel, row_sums=False):
         mode = N.PRUNE_MVUE
         if rand is None:
             rand = _next_philox_state(dense.device)  # uniforms generated inside the kernel
-        if isinstance(rand, tuple):
+        if isinstance(rand, torch.Tensor) and rand.dtype in (torch.int64, torch.uint64) and rand.numel() == 2:
+            if not rand.is_cuda or not rand.is_contiguous():
+                raise RuntimeError("the {seed, offset} state tensor of MVUE24 must be a contiguous device tensor")
+            mode = N.PRUNE_MVUE_SEEDED_DEVICE        # read by the kernel; the call leaves offset += 4 behind
+            rand_t = rand
+        elif isinstance(rand, tuple):
             mode = N.PRUNE_MVUE_SEEDED
             seed_offset = (ctypes.c_uint64 * 2)(int(rand[0]) & (2 ** 64 - 1), int(rand[1]) & (2 ** 64 - 1))
             rand_t = _HostWords(seed_offset)         # read by the library during the call
@@ -322,19 +366,17 @@ class SparseSemiStructuredTensor(torch.Tensor):
     def _set_storage(self, values, meta, shape, layout):
         self._store_values, self._store_meta = values, meta       # flat device tensors
         self._store_shape, self._store_layout = shape, layout     # (m, k) of the untransposed matrix
-        self._canonical = None
-        self._cutlass = None
 
     def _canonical_pair(self):
-        if self._canonical is None:
-            m, n = self._store_shape
-            if self._store_layout == N.COMPRESSED_PANEL:
-                self._canonical = _to_canonical(self._store_values, self._store_meta, m, n)
-            elif self._store_layout == N.COMPRESSED_CUTLASS:
-                self._canonical = (self._store_values.view(m, n // 2), self._converted_meta(N.COMPRESSED_CANONICAL))
-            else:
-                self._canonical = (self._store_values.view(m, n // 2), self._store_meta.view(m, -1))
-        return self._canonical
+        """(values [m, k/2], canonical metadata) of the stored operand.  Made from the storage on every call
+        (views where the storage is canonical, copies otherwise): the storage may be rewritten behind the
+        wrapper's back -- a graph replay recompresses into the same buffers -- so nothing derived is kept."""
+        m, n = self._store_shape
+        if self._store_layout == N.COMPRESSED_PANEL:
+            return _to_canonical(self._store_values, self._store_meta, m, n)
+        if self._store_layout == N.COMPRESSED_CUTLASS:
+            return self._store_values.view(m, n // 2), self._converted_meta(N.COMPRESSED_CANONICAL)
+        return self._store_values.view(m, n // 2), self._store_meta.view(m, -1)
 
     def _converted_meta(self, to_layout):
         """The metadata in another storage form, [m, k/16 | k/32] words (HIP kernel; values untouched)."""
@@ -474,9 +516,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
         if self._store_layout == N.COMPRESSED_CUTLASS:
             m, _ = self._store_shape
             return self._store_meta.view(m, -1)
-        if self._cutlass is None:
-            self._cutlass = self._converted_meta(N.COMPRESSED_CUTLASS)
-        return self._cutlass
+        return self._converted_meta(N.COMPRESSED_CUTLASS)
 
 
 def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = False, MVUE24: bool = False,
@@ -488,7 +528,8 @@ def to_sparse_semi_structured(original_tensor: torch.Tensor, transposed: bool = 
     `mask` (same shape, nonzero = keep) selects explicitly; `MVUE24=True` samples the
     minimum-variance unbiased estimator, taking its uniforms from `rand`: a tensor of the same shape
     (or the packed [m, k/2] form) in [0,1), or a (seed, offset) pair for uniforms generated inside the
-    kernel; when omitted, the pair is taken from torch's generator (torch.manual_seed applies).  `dtype` is the value dtype of the result
+    kernel, or the device-resident pair of mvue_device_state() (then graph replays draw fresh uniforms);
+    when omitted, the pair is taken from torch's generator (torch.manual_seed applies).  `dtype` is the value dtype of the result
     (float16, bfloat16, float8_e4m3fn, float8_e5m2, or int8 for an int8 tensor).  Rows must be a
     multiple of 32, columns of 64 (128 for 8-bit values).  Same signature as the reference's factory (semi_structured.py:575-631)
     plus `rand`.

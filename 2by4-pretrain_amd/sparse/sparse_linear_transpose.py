@@ -16,7 +16,7 @@ from torch import autograd, nn
 
 from .semi_structured import (SparseSemiStructuredTensor, _dense_times_sparse_t, _spmm, to_sparse_semi_structured,
                               to_sparse_semi_structured_pair, to_sparse_semi_structured_with_row_sums)
-from .transposable_semi_structured import TransposableSparse
+from .transposable_semi_structured import TransposableSparse, transposable_mask_
 
 __all__ = ["SparseLinearTranspose", "sparse_linear_transpose"]
 
@@ -96,7 +96,16 @@ class SparseLinearTranspose(nn.Linear):
         else:
             w.mask = w.mask.to(device=w.device)
             if w.counter % w.freq == 0 and w.cnt == 0:
-                _, w.mask = self.transposable_sparse(w)
+                # = `_, w.mask = self.transposable_sparse(w)` (README.md:149-150) with the mask rewritten in place
+                # where the buffer fits: whoever holds the tensor (the masked decay, a recorded graph) sees the
+                # new mask, and the unused pruned copy of w is not written
+                m = w.mask
+                if (torch.is_tensor(m) and m.dtype == torch.bool and m.shape == w.shape and m.stride() == w.stride()
+                        and m.device == w.device and w.is_contiguous() and w.data_ptr() % 16 == 0 and w.shape[1] % 8 == 0
+                        and self.transposable_sparse.abs):
+                    transposable_mask_(w.detach(), m, abs=True)
+                else:
+                    _, w.mask = self.transposable_sparse(w)
             if w.cnt == 0:
                 # = to_sparse_semi_structured(w, mask=w.mask), to_sparse_semi_structured(w.T, mask=w.mask.T)
                 # (README.md:165-166), from one read of w and the mask

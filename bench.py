@@ -231,71 +231,158 @@ def spmm_workload(steps, warmup):
 
 
 # --------------------------------------------------------------------------------------------
+class MlpTrainer:
+    """The training step of BASELINE config 4 -- GPT-2-124M MLP (c_fc d->h, GELU, c_proj h->d), fp16 autocast, mean
+    squared error against a fixed target, fixed loss scale, AdamW -- run eagerly (step) or as replays of HIP graphs
+    that hold one whole step each (capture / replay_step).
+
+    kind  "sparse": SparseLinearTranspose layers (transposable mask refreshed every `freq` optimizer steps, W and
+                    W^T recompressed each step, MVUE24 dW), masked decay alpha = 2e-4 by masked_add_, torch's fused AdamW;
+          "sparse_one_pass": the same with MaskedDecayAdamW (decay folded into the update; eager only);
+          "dense":  nn.Linear layers under autocast, torch's fused AdamW.
+    Graphs: the layer's bookkeeping (`cnt`, `counter`: when to refresh the mask, when to recompress) is host
+    logic that a graph freezes, so two graphs are recorded, a step that refreshes the masks and a step that does
+    not, and replay_step picks by the optimizer step count.  MVUE24 takes its generator state from device memory
+    under capture (sparse.mvue_device_state), so every replay samples afresh; the optimizer keeps its step count
+    on the device (capturable=True)."""
+
+    def __init__(self, kind, tokens=12 * 1024, d=768, h=3072, seed=2, capturable=False, freq=40, loss_scale=4096.0):
+        import sparse
+        self.sparse, self.kind, self.freq, self.loss_scale = sparse, kind, freq, loss_scale
+        dev = torch.device("cuda:0")
+        torch.manual_seed(seed)
+        self.x = torch.randn(tokens, d, device=dev)
+        self.target = torch.randn(tokens, d, device=dev)
+        torch.manual_seed(seed)
+        if kind != "dense":
+            self.fc, self.proj = sparse.SparseLinearTranspose(d, h).to(dev), sparse.SparseLinearTranspose(h, d).to(dev)
+            for layer in (self.fc, self.proj):
+                layer.weight.freq = freq
+        else:
+            self.fc, self.proj = torch.nn.Linear(d, h).to(dev), torch.nn.Linear(h, d).to(dev)
+        for layer in (self.fc, self.proj):
+            torch.nn.init.normal_(layer.weight, std=0.02)
+        self.params = list(self.fc.parameters()) + list(self.proj.parameters())
+        if kind == "sparse_one_pass":      # masked decay folded into the optimizer update
+            self.opt = sparse.MaskedDecayAdamW(self.params, lr=1e-4, weight_decay=0.0, alpha=2e-4)
+        else:
+            self.opt = torch.optim.AdamW(self.params, lr=1e-4, weight_decay=0.0, fused=True, capturable=capturable)
+        self.opt_steps = 0
+        self.graphs = None
+        self.flops = 6 * 2.0 * tokens * d * h          # 3 GEMMs per layer, 2 layers, dense-equivalent
+
+    def _body(self):
+        import torch.nn.functional as F
+        if self.kind != "dense":
+            out = self.proj(F.gelu(self.fc(self.x)))
+        else:
+            with torch.autocast(device_type="cuda", dtype=torch.float16):
+                out = self.proj(F.gelu(self.fc(self.x)))
+        # a mean over tokens x d outputs puts dY near 1e-7, below fp16's normal range: fixed loss scale
+        # (a power of two), gradients unscaled in one multi-tensor launch, in every model
+        loss = F.mse_loss(out.float(), self.target)
+        self.opt.zero_grad(set_to_none=True)
+        (loss * self.loss_scale).backward()
+        torch._foreach_mul_([p.grad for p in self.params], 1.0 / self.loss_scale)
+        if self.kind == "sparse":
+            with torch.no_grad():
+                for p in self.params:
+                    if hasattr(p, "mask") and p.mode == "sparse":
+                        p.grad = p.grad.float()
+                        self.sparse.masked_add_(p.grad.data, p.data, p.mask, alpha=2e-4)
+                        p.cnt = 0
+        self.opt.step()
+        return loss
+
+    def step(self):
+        loss = self._body()
+        self.opt_steps += 1
+        return loss
+
+    def _set_layer_clock(self, counter):
+        for layer in (self.fc, self.proj):
+            if hasattr(layer.weight, "counter"):
+                layer.weight.counter, layer.weight.cnt = counter, 0
+
+    def capture(self, eager_steps=3):
+        """`eager_steps` steps on a side stream (allocator and library warm-up, optimizer state), then the
+        recordings.  Nothing runs during a recording."""
+        assert self.kind in ("sparse", "dense") and self.graphs is None
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(eager_steps):
+                self.step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graphs, self.losses = {}, {}
+        if self.kind == "sparse":
+            gen = torch.cuda.default_generators[0]
+            self.sparse.mvue_device_state(self.x.device, seed=gen.initial_seed(), offset=gen.get_offset())
+        for name in (("refresh", "regular") if self.kind == "sparse" else ("regular",)):
+            self._set_layer_clock(0 if name == "refresh" else 1)        # the mask is searched when counter % freq == 0
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self.losses[name] = self._body()
+            self.graphs[name] = g
+        self._set_layer_clock(self.opt_steps)
+        return self
+
+    def replay_step(self):
+        name = "refresh" if (self.kind == "sparse" and self.opt_steps % self.freq == 0) else "regular"
+        self.graphs[name].replay()
+        self.opt_steps += 1
+        return self.losses[name]
+
+
 def train_workload(steps, warmup):
     """BASELINE config 4: GPT-2-124M MLP (c_fc 768->3072, GELU, c_proj 3072->768) on 12x1024 tokens,
     fp16 autocast, SparseLinearTranspose layers (transposable mask refreshed every 40 optimizer steps,
     W and W^T recompressed each step, MVUE24 dW), masked decay alpha=2e-4, fused AdamW; seed 2.
-    Returns ms/step for the sparse model and for the same MLP with dense nn.Linear layers."""
-    import sparse
-    import torch.nn.functional as F
-    dev = torch.device("cuda:0")
-    torch.manual_seed(2)
-    tokens, d, h = 12 * 1024, 768, 3072
-    x = torch.randn(tokens, d, device=dev)
-    target = torch.randn(tokens, d, device=dev)
-    # a mean over 12288 x 768 outputs puts dY near 1e-7, below fp16's normal range: fixed loss scale
-    # (a power of two), gradients unscaled in one multi-tensor launch, in both models
-    loss_scale = 4096.0
-
-    def build(kind):
-        torch.manual_seed(2)
-        if kind != "dense":
-            fc, proj = sparse.SparseLinearTranspose(d, h).to(dev), sparse.SparseLinearTranspose(h, d).to(dev)
-        else:
-            fc, proj = torch.nn.Linear(d, h).to(dev), torch.nn.Linear(h, d).to(dev)
-        for layer in (fc, proj):
-            torch.nn.init.normal_(layer.weight, std=0.02)
-        params = list(fc.parameters()) + list(proj.parameters())
-        if kind == "sparse_one_pass":      # masked decay folded into the optimizer update
-            return fc, proj, params, sparse.MaskedDecayAdamW(params, lr=1e-4, weight_decay=0.0, alpha=2e-4)
-        return fc, proj, params, torch.optim.AdamW(params, lr=1e-4, weight_decay=0.0, fused=True)
-
-    def run(kind):
-        fc, proj, params, opt = build(kind)
-
-        def step():
-            if kind != "dense":
-                out = proj(F.gelu(fc(x)))
-            else:
-                with torch.autocast(device_type="cuda", dtype=torch.float16):
-                    out = proj(F.gelu(fc(x)))
-            loss = F.mse_loss(out.float(), target)
-            opt.zero_grad(set_to_none=True)
-            (loss * loss_scale).backward()
-            torch._foreach_mul_([p.grad for p in params], 1.0 / loss_scale)
-            if kind == "sparse":
-                with torch.no_grad():
-                    for p in params:
-                        if hasattr(p, "mask") and p.mode == "sparse":
-                            p.grad = p.grad.float()
-                            sparse.masked_add_(p.grad.data, p.data, p.mask, alpha=2e-4)
-                            p.cnt = 0
-            opt.step()
-            return loss
-        settle(lambda i: step())
+    ms/step of the sparse model and of the same MLP with dense nn.Linear layers, each issued eagerly and as
+    replays of whole-step HIP graphs."""
+    def timed(step_fn):
+        settle(lambda i: step_fn())
         for _ in range(warmup):
-            step()
+            step_fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            loss = step()
+            loss = step_fn()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / steps, loss.item()
-    sparse_ms, sparse_loss = run("sparse")
-    dense_ms, dense_loss = run("dense")
-    one_pass_ms, _ = run("sparse_one_pass")
-    flops = 6 * 2.0 * tokens * d * h          # 3 GEMMs per layer, 2 layers, dense-equivalent
-    return sparse_ms, dense_ms, sparse_loss, dense_loss, flops, one_pass_ms
+
+    out = {}
+    for kind in ("sparse", "dense", "sparse_one_pass"):
+        t = MlpTrainer(kind)
+        out[kind + "_ms"], out[kind + "_loss"] = timed(t.step)
+        out["flops"] = t.flops
+        del t
+        torch.cuda.empty_cache()
+    for kind in ("sparse", "dense"):
+        t = MlpTrainer(kind, capturable=True).capture()
+        out[kind + "_graph_ms"], out[kind + "_graph_loss"] = timed(t.replay_step)
+        del t
+        torch.cuda.empty_cache()
+    return out
+
+
+def train_record(r):
+    """The training-step figures as they go into the JSON line."""
+    return {
+        "ms_per_step": round(r["sparse_ms"], 4), "ms_per_step_with_MaskedDecayAdamW": round(r["sparse_one_pass_ms"], 4),
+        "dense_autocast_ms_per_step": round(r["dense_ms"], 4),
+        "speedup_vs_dense_step": round(r["dense_ms"] / r["sparse_ms"], 3),
+        "speedup_vs_dense_step_with_MaskedDecayAdamW": round(r["dense_ms"] / r["sparse_one_pass_ms"], 3),
+        "hip_graph_replay": {
+            "what": "one whole step (forward, backward, masked decay, fused AdamW) per graph replay; the sparse model replays "
+                    "a mask-refresh graph every 40th step and a regular one otherwise; MVUE24 state on the device",
+            "ms_per_step": round(r["sparse_graph_ms"], 4), "dense_autocast_ms_per_step": round(r["dense_graph_ms"], 4),
+            "speedup_vs_dense_step": round(r["dense_graph_ms"] / r["sparse_graph_ms"], 3),
+            "speedup_vs_eager_dense_step": round(r["dense_ms"] / r["sparse_graph_ms"], 3)},
+        "tflops_dense_equivalent": round(r["flops"] / (r["sparse_ms"] * 1e-3) / 1e12, 1),
+        "final_loss": {"sparse (2:4 weights, MVUE24 weight gradients)": r["sparse_loss"],
+                       "dense (unmasked dense model: all weights trained, exact gradients)": r["dense_loss"]}}
 
 
 def int8_workload(steps):
@@ -569,16 +656,15 @@ def main():
         return
 
     if a.workload == "train":
-        sparse_ms, dense_ms, sl, dl, flops, one_pass_ms = train_workload(a.steps, a.warmup)
-        print(json.dumps({
-            "metric": "2:4 sparse MLP training step, dense-equivalent TFLOP/s of its 6 GEMMs", "value": round(flops / (sparse_ms * 1e-3) / 1e12, 2),
-            "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_s": SETTLE_S, "ms_per_step": round(sparse_ms, 4),
+        r = train_workload(a.steps, a.warmup)
+        line = {
+            "metric": "2:4 sparse MLP training step, dense-equivalent TFLOP/s of its 6 GEMMs", "value": round(r["flops"] / (r["sparse_ms"] * 1e-3) / 1e12, 2),
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_s": SETTLE_S, "ms_per_step": round(r["sparse_ms"], 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "BASELINE configs[3]: SparseLinearTranspose GPT-2-124M MLP step, 12288 tokens, 768->3072->768, "
-                                   "masked decay 2e-4, fused AdamW, mask refresh every 40 steps", "seed": 2},
-            "dense_autocast_ms_per_step": round(dense_ms, 4), "speedup_vs_dense_step": round(dense_ms / sparse_ms, 3),
-            "ms_per_step_with_MaskedDecayAdamW": round(one_pass_ms, 4),
-            "final_loss": {"sparse": sl, "dense": dl}}))
+                                   "masked decay 2e-4, fused AdamW, mask refresh every 40 steps", "seed": 2}}
+        line.update(train_record(r))
+        print(json.dumps(line))
         return
 
     if a.workload == "decode":
@@ -665,14 +751,10 @@ def main():
             "speedup_vs_dense_gemm": None if dense_ms is None else round(dense_ms / mm_ms, 3),
             "iteration_ms_with_soft_threshold_and_mvue_compress": round(step_ms, 4), "rel_err_vs_dense_fp32": rel}
         torch.cuda.empty_cache()
-        sparse_ms, dense_step_ms, sl, dl, tf, one_pass_ms = train_workload(a.steps, a.warmup)
         line["train_config4"] = {
             "workload": "BASELINE configs[3]: SparseLinearTranspose GPT-2-124M MLP step, 12288 tokens, 768->3072->768, fp16 autocast, "
-                        "masked decay 2e-4, fused AdamW, mask refresh every 40 steps",
-            "ms_per_step": round(sparse_ms, 4), "ms_per_step_with_MaskedDecayAdamW": round(one_pass_ms, 4),
-            "dense_autocast_ms_per_step": round(dense_step_ms, 4), "speedup_vs_dense_step": round(dense_step_ms / sparse_ms, 3),
-            "speedup_vs_dense_step_with_MaskedDecayAdamW": round(dense_step_ms / one_pass_ms, 3),
-            "tflops_dense_equivalent": round(tf / (sparse_ms * 1e-3) / 1e12, 1), "final_loss": {"sparse": sl, "dense": dl}}
+                        "masked decay 2e-4, fused AdamW, mask refresh every 40 steps"}
+        line["train_config4"].update(train_record(train_workload(a.steps, a.warmup)))
         torch.cuda.empty_cache()
     if not a.no_convert:
         line["conversion_kernels_GBps"] = conversion_kernels()

@@ -4,7 +4,8 @@
  *
  * Conventions
  *   - Every pointer is a DEVICE pointer (HIP); the one exception is `rand` in mode
- *     TF24_PRUNE_MVUE_SEEDED, which points to {seed, offset} in host memory.
+ *     TF24_PRUNE_MVUE_SEEDED, which points to {seed, offset} in host memory
+ *     (TF24_PRUNE_MVUE_SEEDED_DEVICE takes the pair from device memory).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Nothing here
  *     allocates, frees or synchronises: the caller owns every buffer, work is only enqueued.
  *   - Return value: TF24_OK or a negative tf24_status; tf24_last_error() returns a
@@ -56,9 +57,14 @@ typedef enum {
   TF24_PRUNE_MASK = 1,      /* keep what a supplied mask says */
   TF24_PRUNE_MVUE = 2,      /* MVUE24 sampling from a supplied U(0,1) tensor of the dense shape */
   TF24_PRUNE_MVUE_PACKED = 3, /* the same with only the uniforms that are used: a [m, k/2] tensor */
-  TF24_PRUNE_MVUE_SEEDED = 4  /* MVUE24 with uniforms generated in the kernel: `rand` points to two uint64
+  TF24_PRUNE_MVUE_SEEDED = 4, /* MVUE24 with uniforms generated in the kernel: `rand` points to two uint64
                                  values {seed, offset} in HOST memory (read during the call).  The uniforms
                                  are exactly those tf24_mvue_uniforms writes for the same seed and offset. */
+  TF24_PRUNE_MVUE_SEEDED_DEVICE = 5 /* the same with {seed, offset} in DEVICE memory (8-byte aligned), read by the
+                                 kernel when it runs; behind the conversion the call enqueues offset += 4 on
+                                 the same stream, as a host-side generator advances per sampling call.  A call
+                                 recorded into a HIP graph therefore draws fresh uniforms on every replay
+                                 (the host form would replay the values it read at capture). */
 } tf24_prune_mode;
 
 /* GELU is the exact (erf) form, torch.nn.functional.gelu's default; the reference's epilogues stop at SILU */
