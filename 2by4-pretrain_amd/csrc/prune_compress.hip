@@ -259,6 +259,80 @@ prune_compress_row_mag16(const In* __restrict__ dense, int64_t ld, int64_t m, in
   }
 }
 
+// Magnitude mode on 16-bit floats into the PANEL layout: a wave owns 4 adjacent rows x 512 columns.  Each of its
+// four load instructions reads 1 KB of one row; a lane holds the same 8-column unit of the 4 rows, so the metadata
+// words of its quad for the 4 rows are one 16-byte piece of the [k/32][m] word matrix, stored by the quad leader
+// as it is.  (64 rows x 128 columns per block with 256-byte reads per row: 37.0 us at 8192 x 8192 bf16 -> fp16;
+// this kernel 35.5; the same without the exchange of the values, 64-byte pieces per store: 41.4.)
+template <typename In, typename Out>
+__global__ void __launch_bounds__(kThreads)
+prune_compress_row_mag16_panel(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t k,
+                               Out* __restrict__ values, uint8_t* __restrict__ meta) {
+  constexpr int UPP = (128 / (int)sizeof(Out)) / 8;      // units per panel row (8 or 16)
+  constexpr uint32_t kInf = std::is_same<In, f16_t>::value ? 0x7c00u : 0x7f80u;
+  const int64_t upr = k >> 3;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row0 = (int64_t)blockIdx.y * 16 + wave * 4;
+  const int64_t col8 = (int64_t)blockIdx.x * 64 + lane;
+  const bool live = col8 < upr;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 in[4];
+#pragma unroll
+  for (int it = 0; it < 4; it++) {
+    in[it] = u32x4{0, 0, 0, 0};
+    if (live) in[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dense + (row0 + it) * ld + col8 * 8));
+  }
+  // values: a lane's four 8-byte pieces are 64 bytes apart in the panel layout; the wave exchanges them through
+  // a private LDS slice (rows padded by 128 bytes: both halves of a 64-lane read fall on all banks) so that a
+  // store instruction writes, per panel, the 64-byte pieces of the 4 rows: 256 contiguous bytes (two panels, one of 8-bit values)
+  using piece_t = typename vec_bytes<4 * sizeof(Out)>::type;        // a unit's 4 kept values: 8 bytes, or 4 for 8-bit values
+  constexpr int XROW = 64 + 128 / (int)sizeof(piece_t);
+  __shared__ __attribute__((aligned(16))) piece_t s_x[kThreads / 64][4 * XROW];
+  uint32_t words[4];
+#pragma unroll
+  for (int it = 0; it < 4; it++) {
+    const uint32_t w0 = in[it][0], w1 = in[it][1], w2 = in[it][2], w3 = in[it][3];
+    const Top2 t0 = magnitude_top2_16(w0, w1), t1 = magnitude_top2_16(w2, w3);
+    uint32_t n0 = t0.nibble, n1 = t1.nibble;
+    if (max(t0.top_key, t1.top_key) > ((kInf << 2) | 3u)) {          // a NaN in the unit
+      const In* e = reinterpret_cast<const In*>(&in[it]);
+      n0 = encode_nibble(magnitude_mask4(to_float(e[0]), to_float(e[1]), to_float(e[2]), to_float(e[3])));
+      n1 = encode_nibble(magnitude_mask4(to_float(e[4]), to_float(e[5]), to_float(e[6]), to_float(e[7])));
+    }
+    const uint32_t r0 = pick16(w0, w1, n0 & 3u), r1 = pick16(w0, w1, n0 >> 2);
+    const uint32_t r2 = pick16(w2, w3, n1 & 3u), r3 = pick16(w2, w3, n1 >> 2);
+    Pack<Out, 4> out;
+    if constexpr (std::is_same<In, Out>::value) {
+      uint32_t* o = reinterpret_cast<uint32_t*>(out.v);
+      o[0] = (r0 & 0xffffu) | (r1 << 16);
+      o[1] = (r2 & 0xffffu) | (r3 << 16);
+    } else {
+      out.v[0] = from_float<Out>(to_float(In{(uint16_t)r0}));
+      out.v[1] = from_float<Out>(to_float(In{(uint16_t)r1}));
+      out.v[2] = from_float<Out>(to_float(In{(uint16_t)r2}));
+      out.v[3] = from_float<Out>(to_float(In{(uint16_t)r3}));
+    }
+    s_x[wave][it * XROW + lane] = *reinterpret_cast<const piece_t*>(out.v);
+    const uint32_t mbyte = live ? n0 | (n1 << 4) : 0u;
+    uint32_t w = mbyte;
+    w |= __shfl_down(mbyte, 1) << 8;
+    w |= __shfl_down(mbyte, 2) << 16;
+    w |= __shfl_down(mbyte, 3) << 24;
+    words[it] = w;
+  }
+  // lane l' of store instruction i takes row l'/16, unit 16 i + l'%16 (LDS accesses of one wave execute in order: no barrier)
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = lane >> 4, u = 16 * i + (lane & 15);
+    Pack<Out, 4> v;
+    *reinterpret_cast<piece_t*>(v.v) = s_x[wave][r * XROW + u];
+    const int64_t c8 = (int64_t)blockIdx.x * 64 + u;
+    if (c8 < upr) v.store_stream(values + (((c8 / UPP) * m + row0 + r) * UPP + c8 % UPP) * 4);
+  }
+  if (live && (lane & 3) == 0)
+    *reinterpret_cast<uint4*>(meta + panel_meta_offset(col8, row0, m)) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
 // ------------------------------------------------------------------ column-major
 // element (r,c) at c*ld + r.  R = rows per lane = 16 bytes / sizeof(In).
 template <typename In, typename Out, int MODE, typename MaskT>
@@ -454,6 +528,11 @@ int launch(const void* dense, int layout, int64_t ld, int64_t m, int64_t k, cons
       grid = dim3((unsigned)(((k >> 3) + units_per_block - 1) / units_per_block), (unsigned)(m / rows_per_block));
     }
     if constexpr (MODE == TF24_PRUNE_MAGNITUDE && (std::is_same<In, f16_t>::value || std::is_same<In, bf16_t>::value)) {
+      if (panel && m % 16 == 0 && m / 16 <= 65535) {
+        dim3 pgrid((unsigned)(((k >> 3) + 63) / 64), (unsigned)(m / 16));
+        hipLaunchKernelGGL((prune_compress_row_mag16_panel<In, Out>), pgrid, dim3(kThreads), 0, stream, (const In*)dense, ld, m, k, (Out*)values, (uint8_t*)meta);
+        return check_launch("tf24_prune_compress");
+      }
       hipLaunchKernelGGL((prune_compress_row_mag16<In, Out>), grid, dim3(kThreads), 0, stream,
                          (const In*)dense, ld, m, k, (Out*)values, (uint8_t*)meta, contiguous, panel, lpr_shift);
     } else {

@@ -77,10 +77,29 @@ template <> struct mma16<i8_t> {
   }
 };
 
+// Exact (erf) GELU, 0.5 v (1 + erf(v / sqrt 2)), through the complementary error function of |v| / sqrt 2
+// (Abramowitz & Stegun 7.1.26: erfc(z) = t (a1 + t (a2 + t (a3 + t (a4 + t a5)))) exp(-z^2), t = 1 / (1 + p z),
+// absolute error <= 1.5e-7):  with q = erfc(|v| / sqrt 2),  gelu(v) = v - v q / 2 for v >= 0 and v q / 2 below,
+// so the negative tail is not formed as a difference of nearly equal numbers.  One reciprocal, one exponential
+// and nine multiply-adds per element: the library erff costs three times that, which made a GELU output pass
+// slower than a plain one plus a separate GELU kernel.  Agrees with the float32 GELU of torch to 3e-7 absolute.
+__device__ __forceinline__ float gelu_erf(float v) {
+  const float z = __builtin_fabsf(v) * 0.70710678118654752f;
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, z, 1.0f));
+  float poly = __builtin_fmaf(t, 1.061405429f, -1.453152027f);
+  poly = __builtin_fmaf(poly, t, 1.421413741f);
+  poly = __builtin_fmaf(poly, t, -0.284496736f);
+  poly = __builtin_fmaf(poly, t, 0.254829592f);
+  const float q = poly * t * __builtin_amdgcn_exp2f(z * z * -1.4426950408889634f);
+  // |v| clamped where q has long been 0: an infinite v stays infinite (or becomes -0) instead of inf * 0
+  const float h = 0.5f * q * __builtin_amdgcn_fmed3f(v, -65536.0f, 65536.0f);
+  return v >= 0.0f ? v - h : (v < 0.0f ? h : v);
+}
+
 __device__ __forceinline__ float apply_act(float v, int act) {
   if (act == TF24_ACT_RELU) return v > 0.0f ? v : 0.0f;
   if (act == TF24_ACT_SILU) return v / (1.0f + __expf(-v));
-  if (act == TF24_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
+  if (act == TF24_ACT_GELU) return gelu_erf(v);
   return v;
 }
 
@@ -105,12 +124,13 @@ __device__ __forceinline__ int finish_value(int accv, float, const OutT* bias, i
 // bias only, and with both decided at run time.  Left to run-time tests alone, the per-element
 // selects and the inlined SiLU more than triple the time of the pass (21 000 against 6 300 cycles
 // per 256 x 256 tile), which is a tenth of the whole kernel at k = 4096.
-enum { EPI_PLAIN = 0, EPI_BIAS = 1, EPI_RUNTIME = 2 };
+enum { EPI_PLAIN = 0, EPI_BIAS = 1, EPI_RUNTIME = 2, EPI_GELU = 3 };    // GELU: optional bias, then gelu_erf (the MLP's first layer)
 template <int MODE, typename OutT>
 __device__ __forceinline__ float finish_element(float accv, float scale, const OutT* bias, int64_t row, bool row_ok, int act) {
   float v = accv * scale;
   if constexpr (MODE == EPI_BIAS) { if (row_ok) v += to_float(bias[row]); }
   if constexpr (MODE == EPI_RUNTIME) { if (bias && row_ok) v += to_float(bias[row]); v = apply_act(v, act); }
+  if constexpr (MODE == EPI_GELU) { if (bias && row_ok) v += to_float(bias[row]); v = gelu_erf(v); }
   return v;
 }
 
@@ -778,6 +798,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   };
   if (!bias && act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_PLAIN>{});
   else if (act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_BIAS>{});
+  else if (act == TF24_ACT_GELU && !std::is_same<typename mma32<T>::acc4_t, int4v>::value) output_pass(std::integral_constant<int, EPI_GELU>{});
   else output_pass(std::integral_constant<int, EPI_RUNTIME>{});
   if (!has_next) break;
   // ---- the next tile: its first two stages are (about to be) in the buffers nxt and fre

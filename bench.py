@@ -26,17 +26,29 @@ import torch  # noqa: E402
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_DENSE_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA; SMFMAC executes MACs at this rate
 MFMA_DENSE_PEAK_FP8_TFLOPS = 5000.0
-# Bytes that cross the L2 <-> memory-fabric boundary per spmm launch of config 3 (mean of forward and
-# transposed), from two `rocprofv3 --pmc` runs of `bench.py --workload traffic` (FETCH_SIZE, then
-# WRITE_SIZE; KiB per dispatch), each scaled by known / counted bytes of a plain 128 MiB device copy in
-# the same run: FETCH_SIZE 431052 KiB x 2.00 (the counter books this GPU's 128-byte read requests as 64
-# bytes: every streaming kernel of known footprint reads 0.50 of its bytes, and the 32-byte-unit request
-# counter TCC_EA0_RDREQ_DRAM_32B gives the same 883 MB), WRITE_SIZE 120841 KiB x 1.00.  The infinity
-# cache sits behind this boundary, so part of it never reaches HBM.  A profiled constant, not
-# something this run measures: emitted for the config-3 shape only, with its source.
-SPMM_TRAFFIC_PROFILED = int(431052 * 1024 * 2.0 + 120841 * 1024 * 1.0)
-SPMM_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over `bench.py --workload traffic`, factors 2.00 / 1.00 from the "
-                       "128 MiB device copy of the same runs; L2 <-> fabric bytes (infinity cache behind it); summary under profiles/")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "spmm_cfg3_hbm_traffic_counters.md")
+
+
+def profiled_traffic():
+    """Bytes that cross the L2 <-> memory-fabric boundary per spmm launch of config 3 (mean of forward and
+    transposed), as the committed byte-counter summary records them: its `traffic_record:` line holds the
+    FETCH_SIZE / WRITE_SIZE readings (KiB per dispatch) of two `rocprofv3 --pmc` runs of
+    `bench.py --workload traffic`, the factors that a plain device copy of known size gives each counter
+    in the same runs, and the commit whose kernels were profiled.  A profiled figure, not something this
+    run measures: (bytes, source) or (None, reason)."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.startswith("traffic_record:"):
+                    r = json.loads(line[len("traffic_record:"):])
+                    nbytes = int(r["fetch_kib"] * 1024 * r["fetch_factor"] + r["write_kib"] * 1024 * r["write_factor"])
+                    return nbytes, (f"profiles/{os.path.basename(TRAFFIC_PROFILE)}: rocprofv3 --pmc FETCH_SIZE {r['fetch_kib']} KiB x {r['fetch_factor']} + "
+                                    f"WRITE_SIZE {r['write_kib']} KiB x {r['write_factor']} per dispatch over `bench.py --workload traffic`, factors from the "
+                                    f"128 MiB device copy of the same runs; kernels of commit {r['kernel_commit']}; L2 <-> fabric bytes (infinity cache behind it)")
+    except (OSError, ValueError, KeyError) as ex:
+        return None, f"no traffic record ({ex})"
+    return None, "no traffic record in the profile summary"
+
 
 def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -228,6 +240,38 @@ def spmm_workload(steps, warmup):
     flops = 2.0 * M * Nw * K
     return wall_ms, fwd_ms, bwd_ms, dense_fwd_ms, dense_bwd_ms, rel_fwd, rel_bwd, flops, (M, K, Nw)
 
+
+
+def forward_width_sweep(widths=(10240, 12288), steps=50):
+    """The forward product of config 3 with W of other row counts (X[8192,4096] . W^T, W[n,4096]): n = 10240
+    and 12288 are whole numbers of 256-row tiles per compute unit (5 and 6) and multiples of 256, where the
+    dense library is at its best; config 3's own 11008 is neither.  ms, dense-equivalent TFLOP/s and the
+    ratio to the dense GEMM on the masked weights, per width."""
+    import sparse
+    dev = torch.device("cuda:0")
+    M, K = 8192, 4096
+    gen = torch.Generator().manual_seed(3)
+    X = torch.randn(M, K, generator=gen).half().to(dev)
+    rows = []
+    for n in widths:
+        W = (0.02 * torch.randn(n, K, generator=gen)).half().to(dev)
+        ws = sparse.to_sparse_semi_structured(W)
+        wt, Wd = ws.t(), ws.to_dense()
+
+        def timed(fn):
+            settle(lambda i: fn())
+            e = _events(2)
+            e[0].record()
+            for _ in range(steps):
+                fn()
+            e[1].record()
+            torch.cuda.synchronize()
+            return e[0].elapsed_time(e[1]) / steps
+        ours, dense = timed(lambda: torch.mm(X, wt)), timed(lambda: torch.mm(X, Wd.t()))
+        rows.append({"n": n, "ms": round(ours, 4), "tflops_dense_equivalent": round(2.0 * M * n * K / (ours * 1e-3) / 1e12, 1),
+                     "dense_gemm_ms": round(dense, 4), "speedup_vs_dense_gemm": round(dense / ours, 3)})
+        del W, ws, wt, Wd
+    return rows
 
 
 # --------------------------------------------------------------------------------------------
@@ -561,6 +605,96 @@ def cpu_baseline_spmm(threads):
                       f"oracle transposable mask of W {t_tr:.2f} s ({5.0 * Nw * K / t_tr / 1e9:.2f} GB/s algorithmic)"}
 
 
+def cpu_baseline_configs(threads):
+    """The oracle on the host cores beside the other single-GPU configs (2a-e, one training step of config 4,
+    config 5), each on a stated sample -- a slab of rows where the whole matrix would take long -- one warm-up
+    and three timed repetitions, the median; rates are algorithmic bytes (or dense-equivalent flops) of the
+    sample per second."""
+    import oracle
+    torch.set_num_threads(threads)
+
+    def timed(fn, reps=3):
+        fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2]
+
+    out = []
+    gen = torch.Generator().manual_seed(1)
+    rows, k = 8192, 8192                     # config 2 itself
+    n = rows * k
+    W = torch.randn(rows, k, generator=gen).bfloat16()
+    U = torch.rand(rows, k, generator=gen)
+    G = 1e-3 * torch.randn(rows, k, generator=gen)
+    P = W.float()
+    _, tmask = oracle.transposable_mask(W)
+    sample = "the whole 8192 x 8192 matrix of config 2"
+    for name, fn, nbytes in (
+            ("2a magnitude prune+compress bf16 -> f16", lambda: oracle.compress24(W, out_dtype=torch.float16), 3.125 * n),
+            ("2b MVUE24 prune+compress (U float32)", lambda: oracle.mvue24(W, U, out_dtype=torch.float16), 7.125 * n),
+            ("2c transposable mask select", lambda: oracle.transposable_mask(W), 5.0 * n),
+            ("2d soft_threshold24 bf16", lambda: oracle.soft_threshold24(W), 6.0 * n),
+            ("2e masked_add_ f32", lambda: oracle.masked_add(G, P, tmask, alpha=2e-4), 13.0 * n)):
+        t = timed(fn)
+        out.append({"config": name, "seconds": round(t, 4), "value": round(nbytes / t / 1e9, 3), "unit": "GB/s", "sample": sample})
+    del W, U, G, P, tmask
+
+    # config 4: one training step of the MLP in float32 with the oracle's operators (mask search, both compressed
+    # copies, MVUE24 of dY^T for each layer, the six products as dense masked products)
+    tokens, d, h = 12 * 1024, 768, 3072
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(tokens, d, generator=gen)
+    target = torch.randn(tokens, d, generator=gen)
+    w1, w2 = 0.02 * torch.randn(h, d, generator=gen), 0.02 * torch.randn(d, h, generator=gen)
+    u1, u2 = torch.rand(h, tokens, generator=gen), torch.rand(d, tokens, generator=gen)
+
+    def train_step():
+        grads = []
+        m1, m2 = oracle.transposable_mask(w1)[1], oracle.transposable_mask(w2)[1]
+        for w, m in ((w1, m1), (w2, m2)):
+            oracle.compress24(w, mask=m)
+            oracle.compress24(w.t().contiguous(), mask=m.t().contiguous())
+        w1m, w2m = torch.where(m1, w1, torch.zeros(())), torch.where(m2, w2, torch.zeros(()))
+        a = oracle.spmm_ref(x, w1m)
+        hid = torch.nn.functional.gelu(a)
+        y = oracle.spmm_ref(hid, w2m)
+        dy = 2.0 * (y - target) / y.numel()
+        dhid = dy @ w2m
+        dgelu = 0.5 * (1 + torch.erf(a * 0.7071067811865476)) + a * torch.exp(-0.5 * a * a) * 0.3989422804014327
+        for g, inp, u in ((dy, hid, u2), (dhid * dgelu, x, u1)):
+            grads.append(oracle.mvue24_dense(g.t().contiguous(), u) @ inp)
+        for w, g, m in ((w1, grads[1], m1), (w2, grads[0], m2)):
+            oracle.masked_add(g, w, m, alpha=2e-4)
+        return grads
+    t = timed(train_step, reps=1)
+    out.append({"config": "4 one training step (float32, oracle operators; 1 warm-up + 1 timed)", "seconds": round(t, 3),
+                "value": round(6 * 2.0 * tokens * d * h / t / 1e12, 4), "unit": "TFLOP/s dense-equivalent", "sample": "the whole step at full size"})
+    del x, target, w1, w2, u1, u2
+
+    # config 5: MVUE24 of a slab of B, the fp8-quantised product of A against it in float32
+    gen = torch.Generator().manual_seed(5)
+    ra, rb, kk = 4096, 4096, 8192
+    A = torch.randn(ra, kk, generator=gen)
+    B = torch.randn(rb, kk, generator=gen)
+    U = torch.rand(rb, kk, generator=gen)
+    sa, sb = 448.0 / A.abs().max().item(), 224.0 / B.abs().max().item()
+    Aq, Bs = (A * sa).to(torch.float8_e4m3fn), (B * sb).bfloat16()
+
+    def fp8_step():
+        oracle.soft_threshold24(Bs)
+        v, meta, _ = oracle.mvue24(Bs, U, out_dtype=torch.float8_e4m3fn)
+        dense = oracle.decompress24(v, meta).float()
+        return oracle.spmm_ref(Aq.float(), dense)
+    t = timed(fp8_step)
+    out.append({"config": "5 soft threshold + MVUE24 to e4m3 + product (float32 arithmetic on the e4m3 values)", "seconds": round(t, 3),
+                "value": round(2.0 * ra * rb * kk / t / 1e12, 4), "unit": "TFLOP/s dense-equivalent",
+                "sample": f"A rows 0..{ra - 1} of 16384 against B rows 0..{rb - 1} of 8192 (1/8 of the product, half of the conversions)"})
+    return out
+
+
 def host_threads():
     """Threads for the CPU leg: what the host gives this process (its affinity mask, and the
     OMP_NUM_THREADS the box sets), not the machine's core count."""
@@ -713,6 +847,7 @@ def main():
 
     wall_ms, fwd_ms, bwd_ms, dfwd_ms, dbwd_ms, rel_f, rel_b, flops, (M, K, Nw) = spmm_workload(a.steps, a.warmup)
     value = 2 * flops / (wall_ms * 1e-3) / 1e12
+    traffic_bytes, traffic_source = profiled_traffic()
     dom_ms = (fwd_ms + bwd_ms) / 2                       # same kernel, two launches per step
     executed_tflops = (flops / 2) / (dom_ms * 1e-3) / 1e12
     line = {
@@ -724,8 +859,8 @@ def main():
                    "M": M, "K": K, "N": Nw, "seed": 3},
         "roofline": {"bound": "mfma", "kernel": "spmm (SMFMAC)", "achieved": round(executed_tflops, 2),
                      "peak": MFMA_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(executed_tflops / MFMA_DENSE_PEAK_TFLOPS, 4),
-                     "traffic": SPMM_TRAFFIC_PROFILED,
-                     "traffic_source": SPMM_TRAFFIC_SOURCE,
+                     "traffic": traffic_bytes,
+                     "traffic_source": traffic_source,
                      "algorithmic_bytes": M * K * 2 + Nw * K * 9 // 8 + M * Nw * 2,
                      "note": "achieved = executed flops (M*N*K, half the dense-equivalent 2MNK) per launch / HIP-event "
                              "launch time; SMFMAC executes MACs at the dense MFMA rate, so frac also equals "
@@ -738,6 +873,8 @@ def main():
         "rel_err_vs_dense_fp32": {"fwd": rel_f, "transposed": rel_b},
     }
     if not a.no_extra:
+        line["forward_other_widths"] = forward_width_sweep()
+        torch.cuda.empty_cache()
         # the other two single-GPU configs of the baseline, in the same line (each also runs alone
         # with --workload fp8 / train)
         torch.cuda.empty_cache()
@@ -760,6 +897,7 @@ def main():
         line["conversion_kernels_GBps"] = conversion_kernels()
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline_spmm(host_threads())
+        line["cpu_baseline"]["other_configs"] = cpu_baseline_configs(host_threads())
     else:
         line["cpu_baseline"] = None
     print(json.dumps(line))
