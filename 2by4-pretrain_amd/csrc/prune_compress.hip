@@ -129,9 +129,9 @@ prune_compress_row(const In* __restrict__ dense, int64_t ld, int64_t m, int64_t 
           r[0] = r4.v[0]; r[1] = r4.v[1]; r[2] = r4.v[2]; r[3] = r4.v[3];
         } else {
           const float* rp = rs.ptr + row * rs.ld + col8 * 8;
-          Pack<float, 2> ra, rb;                               // the group's two uniforms; read once
-          ra.load_stream(rp);
-          rb.load_stream(rp + 4);
+          Pack<float, 2> ra, rb;                               // the group's two uniforms: the second load meets the first one's line in L1
+          ra.load(rp);
+          rb.load(rp + 4);
           r[0] = ra.v[0]; r[1] = ra.v[1]; r[2] = rb.v[0]; r[3] = rb.v[1];
         }
       }

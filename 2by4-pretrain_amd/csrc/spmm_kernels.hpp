@@ -17,6 +17,7 @@
 #pragma once
 #include "tf24_common.hpp"
 #include <algorithm>
+#include <atomic>
 #include <type_traits>
 
 namespace tf24 {
@@ -895,17 +896,18 @@ TileCost tile_cost(int64_t n_sparse, int64_t k, int64_t n_dense, int64_t workspa
   return {blocks, us};
 }
 
-// compute units of the current device (looked up once per device)
+// compute units of the current device (looked up once per device; the cache is a table of atomics: two threads
+// that meet on an empty entry both look the value up and store the same number)
 inline int compute_units() {
-  static int cached[64];
+  static std::atomic<int> cached[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (!cached[dev]) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (!n) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
 }
 
 template <typename T, typename OutT, typename C>

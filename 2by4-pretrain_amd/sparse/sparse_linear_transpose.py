@@ -28,6 +28,10 @@ class sparse_linear_transpose(autograd.Function):
     and the bias are cast to the compressed copies' dtype and `weight` is left alone.  dW leaves the
     matmul in the master weight's dtype instead of float16 followed by autograd's cast."""
 
+    # True: a 3-d grad_output whose strides are all zero is replaced by ones, as the reference does
+    # (README.md:186-187); False (default): its values are used
+    ones_for_expanded_grad = False
+
     @staticmethod
     def forward(ctx, input, weight, weight_sparse, weight_sparse_T, bias):
         with torch.autocast(device_type="cuda", enabled=False):
@@ -53,7 +57,10 @@ class sparse_linear_transpose(autograd.Function):
             # An expanded scalar gradient (all strides 0: the layer's output fed straight into .sum() or
             # .mean()) is materialised with its values.  The reference replaces a 3-d one by ones
             # (README.md:186-187), which is the same thing after .sum() and scales every gradient by the
-            # element count after .mean(); the values are kept here.
+            # element count after .mean(); the class attribute `ones_for_expanded_grad` switches that
+            # behaviour on for training scripts tuned against it.
+            if sparse_linear_transpose.ones_for_expanded_grad and grad_output.dim() == 3 and grad_output.stride() == (0, 0, 0):
+                grad_output = torch.ones_like(grad_output, memory_format=torch.contiguous_format)
             grad_output = grad_output.reshape(-1, grad_output.shape[-1])
             if grad_output.stride(-1) != 1 or grad_output.stride(0) < grad_output.shape[-1]:
                 grad_output = grad_output.contiguous()
