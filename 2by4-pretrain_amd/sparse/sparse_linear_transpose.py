@@ -54,11 +54,11 @@ class sparse_linear_transpose(autograd.Function):
         input, weight_T, bias = ctx.saved_tensors
         grad_input = grad_weight = grad_bias = None
         with torch.autocast(device_type="cuda", enabled=False):
-            # An expanded scalar gradient (all strides 0: the layer's output fed straight into .sum() or
-            # .mean()) is materialised with its values.  The reference replaces a 3-d one by ones
-            # (README.md:186-187), which is the same thing after .sum() and scales every gradient by the
-            # element count after .mean(); the class attribute `ones_for_expanded_grad` switches that
-            # behaviour on for training scripts tuned against it.
+            # An expanded scalar gradient (all strides 0: the layer's output fed straight into .sum()) is
+            # materialised with its values.  The reference replaces a 3-d one by ones (README.md:186-187), which
+            # is the same thing after a plain .sum() and drops the factor when the sum is scaled (a loss scale,
+            # a weight on the term); the class attribute `ones_for_expanded_grad` switches that behaviour on
+            # for training scripts tuned against it.
             if sparse_linear_transpose.ones_for_expanded_grad and grad_output.dim() == 3 and grad_output.stride() == (0, 0, 0):
                 grad_output = torch.ones_like(grad_output, memory_format=torch.contiguous_format)
             grad_output = grad_output.reshape(-1, grad_output.shape[-1])

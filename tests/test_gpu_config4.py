@@ -258,21 +258,23 @@ def test_mean_reduced_loss_on_the_layer_output(cuda):
 
 def test_reference_switch_for_an_expanded_gradient(cuda):
     """sparse_linear_transpose.ones_for_expanded_grad = True reproduces README.md:186-187: a 3-d grad_output whose
-    strides are all zero (out.sum() / out.mean() taken directly on the layer's output) is replaced by ones, so
-    after .mean() every gradient is the element count times the default behaviour's."""
+    strides are all zero (a scaled out.sum() taken directly on the layer's output) is replaced by ones, so the
+    scale is dropped; by default the gradient's values are used."""
     import sparse
     torch.manual_seed(4)
     layer = sparse.SparseLinearTranspose(256, 512).to(cuda)
     x = torch.randn(4, 128, 256, device=cuda, requires_grad=True)
-    wm = (layer.weight.detach() * 1.0)
     fn = sparse.sparse_linear_transpose
     assert fn.ones_for_expanded_grad is False
-    fn.ones_for_expanded_grad = True
-    try:
-        layer(x).mean().backward()
-    finally:
-        fn.ones_for_expanded_grad = False
-    wm = (layer.weight.detach() * layer.weight.mask).half()
     ones = torch.ones(4 * 128, 512, device=cuda)
-    assert _rel(x.grad.reshape(-1, 256), ones @ wm.float()) < 1e-2
-    assert _rel(layer.bias.grad, ones.sum(0)) < 1e-2
+    for switch, factor in ((False, 3.0), (True, 1.0)):
+        x.grad = layer.weight.grad = layer.bias.grad = None
+        layer.weight.cnt = 0
+        fn.ones_for_expanded_grad = switch
+        try:
+            (layer(x).sum() * 3.0).backward()
+        finally:
+            fn.ones_for_expanded_grad = False
+        wm = (layer.weight.detach() * layer.weight.mask).half()
+        assert _rel(x.grad.reshape(-1, 256), factor * (ones @ wm.float())) < 1e-2, switch
+        assert _rel(layer.bias.grad, factor * ones.sum(0)) < 1e-2, switch
