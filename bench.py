@@ -737,7 +737,7 @@ def traffic_workload(reps=8):
         j = i % nsets
         N.check(lib.tf24_prune_compress(W[j].data_ptr(), N.BF16, N.ROW_MAJOR, k, m, k, N.PRUNE_MAGNITUDE, None, N.U8, 0,
                                         None, 0, values[j].data_ptr(), N.F16, meta[j].data_ptr(), N.COMPRESSED_PANEL, st))
-    known["prune_compress_row"] = {"read": 2 * n, "written": n + n // 8}
+    known["prune_compress_row_mag16_panel"] = {"read": 2 * n, "written": n + n // 8}
     for i in range(reps):
         j = i % nsets
         N.check(lib.tf24_decompress(values[j].data_ptr(), N.F16, meta[j].data_ptr(), N.COMPRESSED_PANEL, m, k, dense[j].data_ptr(), st))
