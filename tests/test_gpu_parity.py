@@ -641,6 +641,46 @@ def test_spmm_chained_tiles_activation_and_scale(cuda, dtype, k, act, scale):
     assert again.equal(out)
 
 
+@pytest.mark.parametrize("dtype,k,act,n,m", [(F16, 1024, None, 4128, 4112), (BF16, 704, "relu", 4128, 4112),
+                                              (E4M3, 1152, "gelu", 4128, 4112), (F16, 576, "silu", 4128, 4112),
+                                              (F16, 768, None, 3072, 12288), (E5M2, 2048, None, 4384, 4352)])
+def test_spmm_partial_last_round_long_k(cuda, dtype, k, act, n, m):
+    """More tiles than compute units with a partial last round and 8 to 32 stages of k (the chained-tile kernel
+    with one to three full rounds before the leftover tiles).  Sums of small integers are exact in float32, so the
+    results must equal the oracle's bit for bit, with bias, scale and activation behind the sum, for k contiguous
+    and k strided dense operands, on a second call, and through the C ABI without a workspace."""
+    import sparse
+    odt = torch.bfloat16 if dtype in FLOAT8 else dtype
+    w = _small_ints((n, k), 84, -2, 3).to(dtype)
+    x = _small_ints((m, k), 85, -2, 3).to(dtype)
+    bias = (_small_ints((n,), 86) * 0.5).to(odt)
+    mask = oracle.prune24_mask(w.float())
+    pre = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(()))) * 0.5 + bias.float()
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    xg = x.to(cuda)
+    run = lambda xin: sparse.sparse_semi_structured_linear(xin, s, bias_opt=bias.to(cuda), activation_opt=act, out_dtype=odt, scale=0.5)
+    out = run(xg)
+    got = out.float().cpu()
+    if act in (None, "relu"):
+        want = pre if act is None else pre.clamp_min(0)
+        assert got.equal(want.to(odt).float())
+    else:
+        want = torch.nn.functional.silu(pre) if act == "silu" else torch.nn.functional.gelu(pre)
+        ulp = 2.0 ** -8 if odt == torch.bfloat16 else 2.0 ** -11
+        err = (got - want).abs()
+        assert bool((err <= 2e-3 + (2e-3 + ulp) * want.abs()).all()), float(err.max())
+    assert run(xg).equal(out)
+    if dtype not in FLOAT8:
+        assert run(maybe_t(xg, True)).equal(out)                # k strided dense operand
+    y = torch.empty((m, n), dtype=odt, device=cuda)
+    N = sparse._native
+    N.check(N.lib().tf24_spmm(s._store_values.data_ptr(), s._store_meta.data_ptr(), s._store_layout, N.operand_code(s._store_values.dtype), n, k,
+                              xg.data_ptr(), N.ROW_MAJOR, k, m, y.data_ptr(), N.operand_code(odt), N.COL_MAJOR, n,
+                              bias.to(cuda).data_ptr(), 0.5, {None: N.ACT_NONE, "relu": N.ACT_RELU, "silu": N.ACT_SILU, "gelu": N.ACT_GELU}[act],
+                              None, 0, N.stream_ptr()))
+    assert y.equal(out)
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16, E4M3, E5M2])
 def test_spmm_tiled_all_operand_positions(cuda, dtype):
     """Shapes large enough for the tiled kernel, with partial tiles: both operand positions, both
