@@ -313,6 +313,16 @@ struct TileCfgT {
   static constexpr int NA = BI * A_ROW / 1024 / NW;   //                                 A values
 };
 using TiledCfg = TileCfgT<4, 2>;
+// The same 256 x 256 tile on four waves, one per SIMD, each computing 128 x 128 with 256 accumulator registers
+// (the 512-register budget of a wave that has its SIMD to itself).  Every fragment read from LDS then feeds four
+// matrix instructions instead of two or four: 100 KB of fragment reads per stage instead of 132 KB.  In cycles the
+// two forms are equal (the matrix pipes are busy for 0.72 of them on config 3 either way), but the kernel runs
+// against the power limit, and with 29 % fewer LDS cycles the clock settles higher: 2.5 % less time on config 3,
+// 3 to 4.6 % on the fp8 product of config 5.  With few stages per tile the longer prologue and output pass of a
+// 4-wave workgroup cost more than that (12 stages: 8 % slower), so only chained tiles of kWave4MinStages or more
+// stages take this form.
+using Wave4Cfg = TileCfgT<2, 4>;
+constexpr int kWave4MinStages = 48;
 // 256 x 64 tiles, two waves: for dense operands of at most 64 columns (a few dozen tokens), where a
 // 256-wide tile would copy and multiply clamped columns.  26 KB per stage, two blocks per CU.
 using SlimCfg = TileCfgT<1, 2>;
@@ -566,8 +576,39 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // (into the buffer at LDS address dst); with `reads`, the fragments of step rstep of the buffer at
   // offset src go into the other register set.
   constexpr int PER_SLOT = (NCOPY + 2 * C::TI - 1) / (2 * C::TI);
+  // copies of a stage issued during the first of its two steps (the rest during the second)
+  constexpr int FIRST_HALF_COPIES = C::NW == 4 ? (NCOPY + 1) / 2 : (C::TI * PER_SLOT < NCOPY ? C::TI * PER_SLOT : NCOPY);
   auto mma_step = [&](int set, int half, bool copies, int pst, uint32_t dst, bool reads, uint32_t src, int rstep) {
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (C::NW == 4) {
+      // One wave per SIMD: no other wave fills the matrix pipe while this one issues reads and copies, so they go
+      // one by one behind every matrix instruction instead of in a block behind a row of them (in blocks: 5 % slower
+      // than the 8-wave form instead of 2.5 % faster).  Ending the reads a few instructions before the step does, so
+      // that the stage barrier finds them landed, changes nothing measurable.
+      constexpr int SLOTS = C::TI * C::TJ;
+      static_assert(!B_KSTRIDED, "the 4-wave form is built for a k-contiguous dense operand (with the transposing reads it spills)");
+#pragma unroll
+      for (int ti = 0; ti < C::TI; ti++) {
+#pragma unroll
+        for (int tj = 0; tj < C::TJ; tj++) {
+          const int4v lo = bf[set][tj][0], hi = bf[set][tj][1];
+          const int8v bfrag = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          acc[ti][tj] = mma32<T>::run(af[set][ti], bfrag, acc[ti][tj], idx[set][ti]);
+          __builtin_amdgcn_sched_barrier(0);
+          const int n = ti * C::TJ + tj;
+          if (reads) {
+#pragma unroll
+            for (int u = 0; u < (N_READS + SLOTS - 1) / SLOTS; u++)
+              if (n * N_READS / SLOTS + u < (n + 1) * N_READS / SLOTS) read_one(set ^ 1, n * N_READS / SLOTS + u, src, rstep);
+          }
+#pragma unroll
+          for (int q = 0; q < NCOPY; q++)
+            if ((q * 2 * SLOTS) / NCOPY == half * SLOTS + n && copies) issue_one(q, pst, dst);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int ti = 0; ti < C::TI; ti++) {
 #pragma unroll
@@ -634,7 +675,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     for (int n = 0; n < N_READS; n++) read_one(0, n, cur, 0);
     if (more) {
 #pragma unroll
-      for (int q = 0; q < C::TI * PER_SLOT && q < NCOPY; q++) issue_one(q, 2, smem_at + fre);
+      for (int q = 0; q < FIRST_HALF_COPIES; q++) issue_one(q, 2, smem_at + fre);
     }
     mma_step(0, 1, more, 2, smem_at + fre, true, cur, 1);
     if (PERSIST && chained) wait_reads_and_barrier();
@@ -926,6 +967,14 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   const bool jm = c_layout == TF24_COL_MAJOR;
   auto launch = [&](auto c_jmajor, auto b_kstrided) {
     if constexpr (C::BJ == 256 && sizeof(OutT) == 2 && decltype(c_jmajor)::value) {
+      if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value) {
+        if (persist && k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages) {      // long chained tiles: the 4-wave form
+          hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true>), grid, dim3(Wave4Cfg::THREADS), 0, s,
+                             (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                             (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
+          return;
+        }
+      }
       if (persist) {
         hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, true>), grid, dim3(C::THREADS), 0, s,
                            (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
