@@ -319,10 +319,10 @@ using TiledCfg = TileCfgT<4, 2>;
 // two forms are equal (the matrix pipes are busy for 0.72 of them on config 3 either way), but the kernel runs
 // against the power limit, and with 29 % fewer LDS cycles the clock settles higher: 2.5 % less time on config 3,
 // 3 to 4.6 % on the fp8 product of config 5.  With few stages per tile the longer prologue and output pass of a
-// 4-wave workgroup cost more than that (12 stages: 8 % slower), so only chained tiles of kWave4MinStages or more
-// stages take this form.
+// 4-wave workgroup cost more than that (12 stages: 8 % slower; 24: equal; 32: 0.6 to 1.3 % faster), so only chained
+// tiles of kWave4MinStages or more stages take this form.
 using Wave4Cfg = TileCfgT<2, 4>;
-constexpr int kWave4MinStages = 48;
+constexpr int kWave4MinStages = 32;
 // 256 x 64 tiles, two waves: for dense operands of at most 64 columns (a few dozen tokens), where a
 // 256-wide tile would copy and multiply clamped columns.  26 KB per stage, two blocks per CU.
 using SlimCfg = TileCfgT<1, 2>;

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "tf24_mvue24_dense": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _i64, _p, _p]),
     "tf24_masked_add": (_i, [_p, _i, _p, _i, _p, _i, _i64, _f, _p]),
     "tf24_adamw_masked_decay": (_i, [_p, _p, _i, _p, _p, _p, _i, _i64, _d, _d, _d, _d, _d, _d, _i64, _p]),
+    "tf24_adamw_masked_decay_device_step": (_i, [_p, _p, _i, _p, _p, _p, _i, _i64, _d, _d, _d, _d, _d, _d, _p, _p]),
     "tf24_gelu_glu_forward": (_i, [_p, _i, _i, _i64, _i64, _i64, _p, _i64, _p]),
     "tf24_gelu_glu_backward": (_i, [_p, _i64, _p, _i, _i, _i64, _i64, _i64, _p, _i64, _p]),
     "tf24_adamw_step": (_i, [_p, _p, _i, _p, _p, _p, _p, _i64, _d, _d, _d, _d, _d, _i64, _p, _i, _p]),

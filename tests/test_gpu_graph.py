@@ -106,19 +106,21 @@ def test_mvue_in_a_graph_draws_fresh_uniforms_on_every_replay(cuda):
     assert int(state.cpu()[1]) == offset + 16
 
 
-def test_whole_training_step_replayed_from_graphs_equals_eager_steps(cuda):
+@pytest.mark.parametrize("kind", ["sparse", "sparse_one_pass"])
+def test_whole_training_step_replayed_from_graphs_equals_eager_steps(cuda, kind):
     """The config-4 training step (here 1024 tokens, 256 -> 512 -> 256, mask refresh every 4 steps) recorded into two
     HIP graphs (a step that refreshes the transposable masks, a step that does not) and replayed for 9 steps,
     against the same model stepped eagerly: masks, weights, biases and optimizer moments bit-equal after every
     step.  Both models draw MVUE24 uniforms from the same (seed, offset) sequence -- the eager one from torch's
     generator on the host, the replayed one from the state in device memory -- so any node of the graph that
-    misbehaved on a replay (a memset node, a frozen offset, a stale mask buffer) would show."""
+    misbehaved on a replay (a memset node, a frozen offset, a stale mask buffer) would show.  kind "sparse": masked_add_
+    + torch's fused AdamW; "sparse_one_pass": MaskedDecayAdamW with its step count on the device."""
     import bench
     kw = dict(tokens=1024, d=256, h=512, freq=4, capturable=True)
-    eager = bench.MlpTrainer("sparse", **kw)
+    eager = bench.MlpTrainer(kind, **kw)
     for _ in range(3):
         eager.step()
-    graphed = bench.MlpTrainer("sparse", **kw).capture(eager_steps=3)
+    graphed = bench.MlpTrainer(kind, **kw).capture(eager_steps=3)
     assert graphed.opt_steps == 3 and set(graphed.graphs) == {"refresh", "regular"}
     losses = []
     for step in range(3, 12):

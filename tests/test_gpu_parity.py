@@ -648,7 +648,7 @@ def test_spmm_chained_tiles_activation_and_scale(cuda, dtype, k, act, scale):
                                               (E4M3, 6144, "relu", 4128, 4112), (E5M2, 6272, "silu", 4384, 4352)])
 def test_spmm_partial_last_round_long_k(cuda, dtype, k, act, n, m):
     """More tiles than compute units with a partial last round and 8 to 49 stages of k (the chained-tile kernel
-    with one to three full rounds before the leftover tiles; from 48 stages on in its 4-wave form).  Sums of small integers are exact in float32, so the
+    with one to three full rounds before the leftover tiles; from 32 stages on in its 4-wave form).  Sums of small integers are exact in float32, so the
     results must equal the oracle's bit for bit, with bias, scale and activation behind the sum, for k contiguous
     and k strided dense operands, on a second call, and through the C ABI without a workspace."""
     import sparse

@@ -264,6 +264,57 @@ def test_masked_decay_adamw_kernel(cuda, gdt):
         assert torch.allclose(plain.detach(), ref_plain.detach(), rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+def test_masked_decay_adamw_step_count_on_the_device(cuda, gdt):
+    """capturable=True: the step count is an int64 in device memory and the bias corrections 1 - beta^step are
+    formed by the kernel.  Twelve updates must leave parameters and moments bit-equal to the optimizer with the
+    count on the host (same double-precision formulas, rounded to float32 at the same places), for a masked
+    parameter and an unmasked one with an odd length; then a single update recorded into a HIP graph and replayed
+    three times must continue the same sequence (a recording with the count frozen in it would not)."""
+    import sparse
+    g = torch.Generator().manual_seed(33)
+    hyp = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1, alpha=2e-4)
+    p0, q0 = torch.randn(96, 200, generator=g), torch.randn(1003, generator=g)
+    mask = (torch.rand(96, 200, generator=g) > 0.5).to(cuda)
+    models = []
+    for capturable in (False, True):
+        par, plain = torch.nn.Parameter(p0.clone().to(cuda)), torch.nn.Parameter(q0.clone().to(cuda))
+        par.mask, par.mode, par.cnt = mask, "sparse", 0
+        if gdt != torch.float32:
+            par.grad_dtype = plain.grad_dtype = None
+        par.grad, plain.grad = torch.zeros(96, 200, device=cuda, dtype=gdt), torch.zeros(1003, device=cuda, dtype=gdt)
+        models.append((par, plain, sparse.MaskedDecayAdamW([par, plain], capturable=capturable, **hyp)))
+    (hp, hq, hopt), (dp, dq, dopt) = models
+
+    def same(step):
+        for a, b in ((hp, dp), (hq, dq)):
+            assert torch.equal(a, b), step
+            assert torch.equal(hopt.state[a]["exp_avg"], dopt.state[b]["exp_avg"]), step
+            assert torch.equal(hopt.state[a]["exp_avg_sq"], dopt.state[b]["exp_avg_sq"]), step
+            assert int(dopt.state[b]["step"]) == hopt.state[a]["step"] == step
+
+    grads = [(torch.randn(96, 200, generator=g).to(gdt).to(cuda), torch.randn(1003, generator=g).to(gdt).to(cuda)) for _ in range(15)]
+    for step in range(1, 13):
+        for par, plain, opt in models:
+            par.grad.copy_(grads[step - 1][0]); plain.grad.copy_(grads[step - 1][1])
+            opt.step()
+        same(step)
+    assert dopt.state[dp]["step"].is_cuda and dopt.state[dp]["step"].dtype == torch.int64
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        dopt.step()
+    for step in range(13, 16):
+        dp.grad.copy_(grads[step - 1][0]); dq.grad.copy_(grads[step - 1][1])
+        graph.replay()
+        hp.grad.copy_(grads[step - 1][0]); hq.grad.copy_(grads[step - 1][1])
+        hopt.step()
+        torch.cuda.synchronize()
+        same(step)
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.float16, 1e-3), (torch.bfloat16, 8e-3)])
 @pytest.mark.parametrize("shape", [(4, 32, 256), (3, 5, 24), (2, 7, 10), (1, 1, 2)])
 @pytest.mark.parametrize("transposed", [False, True])
