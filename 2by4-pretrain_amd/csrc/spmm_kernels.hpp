@@ -317,8 +317,9 @@ using TiledCfg = TileCfgT<4, 2>;
 // (the 512-register budget of a wave that has its SIMD to itself).  Every fragment read from LDS then feeds four
 // matrix instructions instead of two or four: 100 KB of fragment reads per stage instead of 132 KB.  In cycles the
 // two forms are equal (the matrix pipes are busy for 0.72 of them on config 3 either way), but the kernel runs
-// against the power limit, and with 29 % fewer LDS cycles the clock settles higher: 2.5 % less time on config 3,
-// 3 to 4.6 % on the fp8 product of config 5.  With few stages per tile the longer prologue and output pass of a
+// against the power limit, and with 29 % fewer LDS cycles the clock settles higher: 0.5 to 2.7 % less time on the
+// fp16 products of 8192 x 4096 x 11008 (more on boxes with less power headroom), 2.8 to 4.6 % on the fp8 product of
+// 16384 x 8192 x 8192.  With few stages per tile the longer prologue and output pass of a
 // 4-wave workgroup cost more than that (12 stages: 8 % slower; 24: equal; 32: 0.6 to 1.3 % faster), so only chained
 // tiles of kWave4MinStages or more stages take this form.
 using Wave4Cfg = TileCfgT<2, 4>;
@@ -583,7 +584,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     if constexpr (C::NW == 4) {
       // One wave per SIMD: no other wave fills the matrix pipe while this one issues reads and copies, so they go
       // one by one behind every matrix instruction instead of in a block behind a row of them (in blocks: 5 % slower
-      // than the 8-wave form instead of 2.5 % faster).  Ending the reads a few instructions before the step does, so
+      // than the 8-wave form instead of faster).  Ending the reads a few instructions before the step does, so
       // that the stage barrier finds them landed, changes nothing measurable.
       constexpr int SLOTS = C::TI * C::TJ;
       static_assert(!B_KSTRIDED, "the 4-wave form is built for a k-contiguous dense operand (with the transposing reads it spills)");
