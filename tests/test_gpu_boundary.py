@@ -236,3 +236,52 @@ def test_product_from_reference_ordered_metadata(cuda, dtype, n, k, j):
     finally:
         cls._CUTLASS_METADATA = False
     assert fresh.indices().cpu().equal(meta)
+
+
+@pytest.mark.parametrize("dtype,n,k,j,sparse_first", [
+    (torch.float16, 96, 256, 8, False),            # one-pass kernel for a few dense columns
+    (torch.float16, 352, 640, 48, False),          # 256 x 64 tiles
+    (torch.bfloat16, 352, 640, 120, False),        # 256 x 128 tiles
+    (torch.float16, 352, 640, 296, False),         # 256 x 256 tiles, one workgroup per tile
+    (torch.float16, 352, 640, 296, True),          # i-major output, k strided dense operand
+    (torch.float16, 256, 4096, 264, False),        # k pieces through the workspace
+    (torch.bfloat16, 4128, 320, 4112, False),      # chained tiles, 8 waves
+    (torch.float16, 4128, 2112, 4112, False),      # chained tiles, 4 waves (33 stages)
+    (torch.float8_e4m3fn, 4128, 4224, 4112, False),
+    (torch.float8_e4m3fn, 352, 640, 304, False)])
+def test_spmm_padded_leading_dimensions(cuda, dtype, n, k, j, sparse_first):
+    """tf24_spmm through the C ABI with ldb and ldc larger than the rows they address (operands that are slices of
+    wider buffers): the product must equal the contiguous one bit for bit and nothing outside the [rows, cols]
+    window of the output buffer may be written (it is pre-filled with a sentinel)."""
+    import sparse
+    N = sparse._native
+    odt = torch.bfloat16 if dtype == torch.float8_e4m3fn else dtype
+    pad_b, pad_c = 16 * 3, 8 * 5
+    w = _small_ints((n, k), 91, -2, 3).to(dtype)
+    x = _small_ints((j, k), 92, -2, 3).to(dtype)
+    bias = (_small_ints((n,), 93) * 0.5).to(odt).to(cuda)
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    mask = oracle.prune24_mask(w.float())
+    want = (oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(()))) + bias.float().cpu()).to(odt)     # [j, n]
+    if sparse_first:
+        # S @ dense with dense [k, j] row-major in a wider buffer (k strided), output [n, j] row-major in a wider buffer
+        wide_b = torch.zeros(k, j + pad_b, dtype=dtype, device=cuda)
+        wide_b[:, :j] = x.to(cuda).t()
+        wide_c = torch.full((n, j + pad_c), 7.0, dtype=odt, device=cuda)
+        b_layout, ldb, c_layout, ldc = N.COL_MAJOR, j + pad_b, N.ROW_MAJOR, j + pad_c
+        want = want.t()
+    else:
+        wide_b = torch.zeros(j, k + pad_b, dtype=dtype, device=cuda)
+        wide_b[:, :k] = x.to(cuda)
+        wide_c = torch.full((j, n + pad_c), 7.0, dtype=odt, device=cuda)
+        b_layout, ldb, c_layout, ldc = N.ROW_MAJOR, k + pad_b, N.COL_MAJOR, n + pad_c
+    code = N.operand_code(dtype)
+    ws_bytes = N.lib().tf24_spmm_workspace_bytes(code, n, k, j)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=cuda)
+    N.check(N.lib().tf24_spmm(s._store_values.data_ptr(), s._store_meta.data_ptr(), s._store_layout, code, n, k,
+                              wide_b.data_ptr(), b_layout, ldb, j, wide_c.data_ptr(), N.operand_code(odt), c_layout, ldc,
+                              bias.data_ptr(), 1.0, N.ACT_NONE, ws.data_ptr() if ws_bytes else None, ws_bytes, N.stream_ptr()))
+    torch.cuda.synchronize()
+    rows, cols = want.shape
+    assert wide_c[:, :cols].float().cpu().equal(want.float())
+    assert bool((wide_c[:, cols:] == 7.0).all())
