@@ -641,7 +641,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     }
   };
   static_assert(C::STEPS == 2, "the pipeline below is written for two instruction steps per stage");
-  static_assert(!PERSIST || (C_JMAJOR && sizeof(OutT) == 2), "chained tiles rely on the wait inside the j-major 16-bit output pass");
+  static_assert(!PERSIST || C_JMAJOR, "chained tiles rely on the wait inside the j-major output passes");
   auto stage_barrier = [&](bool more) {          // B(st+1): only this wave's copies of stage st+2 may still fly
     if (!more) wait_copies_and_barrier<0>();
     else if (MWAVES == C::NW || has_meta) wait_copies_and_barrier<NCOPY>();
@@ -771,6 +771,40 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
           // the next tile's first two stages (issued one and two stages ago) have to be in LDS before this
           // wave's first store joins the outstanding operations
           if (PERSIST && tj == 0 && ip == 0 && has_next) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  #pragma unroll
+          for (int it = 0; it < 4; it++) {
+            const int jl = it * 8 + rr;
+            const int64_t jrow = j0 + wj * C::WJ + tj * 32 + jl;
+            const int4v v = *reinterpret_cast<const int4v*>(stage + jl * 128 + ((chr ^ (jl & 7)) * 16));
+            if (jrow < n_dense && icol < n_sparse) __builtin_nontemporal_store(v, reinterpret_cast<int4v*>(c + jrow * ldc + icol));
+          }
+        }
+      }
+    } else if constexpr (C_JMAJOR && sizeof(OutT) == 4) {
+      // j-major 32-bit output (float32 from 8-bit operands, int32 from int8: the reference's output types for
+      // them): the same staging with 32(j) x 32(i) pieces -- a lane's four consecutive i are one 16-byte chunk of
+      // a 128-byte row -- so that the stores are full 128-byte row segments instead of 32-byte ones.
+      uint8_t* stage = smem + cur + wave * 4096;
+      const int rr = lane >> 3, chr = lane & 7;
+  #pragma unroll
+      for (int tj = 0; tj < C::TJ; tj++) {
+  #pragma unroll
+        for (int ti = 0; ti < C::TI; ti++) {
+  #pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
+            typedef OutT out4v __attribute__((ext_vector_type(4)));
+            out4v o;
+  #pragma unroll
+            for (int r = 0; r < 4; r++) {
+              o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
+            }
+            const int ch = g * 2 + lh;
+            *reinterpret_cast<out4v*>(stage + l32 * 128 + ((ch ^ (l32 & 7)) * 16)) = o;
+          }
+          const int64_t icol = i0 + wi * C::WI + ti * 32 + chr * 4;
+          // (chained tiles: see the 16-bit pass)
+          if (PERSIST && tj == 0 && ti == 0 && has_next) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   #pragma unroll
           for (int it = 0; it < 4; it++) {
             const int jl = it * 8 + rr;
@@ -962,12 +996,12 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   // More tiles than compute units and no k pieces: one workgroup per compute unit walks its tiles in
   // one pipeline (the next tile's operands arrive while the current one is written out).
   const int cu_slots = compute_units() / 8;
-  const bool persist = C::BJ == 256 && sizeof(OutT) == 2 && c_layout == TF24_COL_MAJOR && splits == 1 &&
+  const bool persist = C::BJ == 256 && c_layout == TF24_COL_MAJOR && splits == 1 &&
                        k * (int64_t)sizeof(T) / C::KB >= 4 && per_xcd > cu_slots && cu_slots > 0;
   dim3 grid((unsigned)((persist ? cu_slots : per_xcd) * 8));
   const bool jm = c_layout == TF24_COL_MAJOR;
   auto launch = [&](auto c_jmajor, auto b_kstrided) {
-    if constexpr (C::BJ == 256 && sizeof(OutT) == 2 && decltype(c_jmajor)::value) {
+    if constexpr (C::BJ == 256 && decltype(c_jmajor)::value) {
       if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value) {
         if (persist && k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages) {      // long chained tiles: the 4-wave form
           hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true>), grid, dim3(Wave4Cfg::THREADS), 0, s,

@@ -1032,3 +1032,43 @@ def test_narrowing_edge_values(cuda):
         assert bool((got[nan].float() != got[nan].float()).all()), odt          # NaN stays NaN (payloads are not compared for 16-bit types)
         if odt in FLOAT8:
             assert gb[nan].equal(wb[nan]), odt                                   # one NaN byte per sign, as torch's
+
+
+@pytest.mark.parametrize("dtype,k,act", [(E4M3, 512, None), (E4M3, 4224, "relu"), (E5M2, 640, "silu"), (F16, 320, "relu"),
+                                         (BF16, 2112, None), (torch.int8, 512, None), (torch.int8, 4224, "relu")])
+def test_spmm_chained_tiles_32bit_output(cuda, dtype, k, act):
+    """More tiles than compute units with a 32-bit output -- float32 from 8-bit operands and int32 from int8, the
+    output types the reference gives them (.cu:729, 772; .cu:594-637), float32 from 16-bit ones -- on the chained-tile
+    kernel (4 to 5 stages: 8 waves; 33 stages: 4 waves) with its staged 32-bit output pass: 17 x 17 tiles with partial
+    edges, bias, activation, against the oracle on exact data, and a second call."""
+    import sparse
+    n, m = 4128, 4112
+    if dtype == torch.int8:
+        w, x = _int8((n, k), 121, -20, 21), _int8((m, k), 122, -20, 21)
+        bias = torch.randint(-1000, 1000, (n,), generator=torch.Generator().manual_seed(123), dtype=torch.int64).int()
+        mask = oracle.prune24_mask(w.float())
+        want = oracle.spmm_ref_int(x, torch.where(mask, w, torch.zeros_like(w))) + bias
+        if act == "relu":
+            want = want.clamp_min(0)
+        s = sparse.to_sparse_semi_structured(w.to(cuda), dtype=torch.int8)
+        out = sparse.sparse_semi_structured_linear(x.to(cuda), s, bias_opt=bias.to(cuda), activation_opt=act)
+        assert out.dtype == torch.int32 and out.shape == (m, n)
+        assert out.cpu().equal(want.int())
+        assert sparse.sparse_semi_structured_linear(x.to(cuda), s, bias_opt=bias.to(cuda), activation_opt=act).equal(out)
+        return
+    w = _small_ints((n, k), 124, -2, 3).to(dtype)
+    x = _small_ints((m, k), 125, -2, 3).to(dtype)
+    bias = _small_ints((n,), 126) * 0.5
+    mask = oracle.prune24_mask(w.float())
+    pre = oracle.spmm_ref(x.float(), torch.where(mask, w.float(), torch.zeros(()))) * 0.25 + bias
+    s = sparse.to_sparse_semi_structured(w.float().to(cuda), dtype=dtype)
+    run = lambda: sparse.sparse_semi_structured_linear(x.to(cuda), s, bias_opt=bias.to(cuda), activation_opt=act, out_dtype=torch.float32, scale=0.25)
+    out = run()
+    assert out.dtype == torch.float32 and out.shape == (m, n)
+    got = out.cpu()
+    if act in (None, "relu"):
+        assert got.equal(pre if act is None else pre.clamp_min(0))
+    else:
+        want = torch.nn.functional.silu(pre)
+        assert bool(((got - want).abs() <= 2e-6 + 2e-6 * want.abs()).all())
+    assert run().equal(out)
