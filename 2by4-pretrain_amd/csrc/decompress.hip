@@ -136,14 +136,31 @@ extern "C" int tf24_repack_to(const void* values_in, const void* meta_in, int dt
   auto known = [](int l) { return l == TF24_COMPRESSED_CANONICAL || l == TF24_COMPRESSED_PANEL || l == TF24_COMPRESSED_CUTLASS; };
   if (!known(from_layout) || !known(to_layout) || from_layout == to_layout)
     return fail(TF24_ERR_ARG, "%s: bad pair of compressed layouts (%d -> %d)", fn, from_layout, to_layout);
-  if (from_layout != TF24_COMPRESSED_CUTLASS && to_layout != TF24_COMPRESSED_CUTLASS)
+  if (from_layout != TF24_COMPRESSED_CUTLASS && to_layout != TF24_COMPRESSED_CUTLASS && values_out && meta_out)
     return tf24_repack(values_in, meta_in, dtype, m, k, from_layout, values_out, meta_out, stream);
   if (dtype != TF24_F16 && dtype != TF24_BF16 && !is_8bit(dtype)) return fail(TF24_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
   const int64_t kp = is_8bit(dtype) ? 128 : 64;
+  if (from_layout != TF24_COMPRESSED_CUTLASS && to_layout != TF24_COMPRESSED_CUTLASS && values_out && !meta_out) {
+    // canonical <-> panel, values only
+    if (m <= 0 || k <= 0 || k % kp) return fail(TF24_ERR_SHAPE, "%s: k=%lld must be a positive multiple of %lld", fn, (long long)k, (long long)kp);
+    if (!values_in || values_in == values_out) return fail(TF24_ERR_ARG, "%s: null pointer or in-place conversion", fn);
+    if (((uintptr_t)values_in | (uintptr_t)values_out) % 16) return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte aligned", fn);
+    const int64_t panels = k / kp, chunks = (panels + 7) / 8, vblocks = chunks * ((m + 7) / 8);
+    if (vblocks > 0x7fffffffLL) return fail(TF24_ERR_SHAPE, "%s: matrix too large", fn);
+    const bool to_panel = to_layout == TF24_COMPRESSED_PANEL;
+    if (kp == 128)
+      hipLaunchKernelGGL(repack_kernel<16>, dim3((unsigned)vblocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint8_t*)values_in,
+                         (const uint8_t*)nullptr, m, panels, (uint32_t)chunks, to_panel, (uint8_t*)values_out, (uint8_t*)nullptr);
+    else
+      hipLaunchKernelGGL(repack_kernel<8>, dim3((unsigned)vblocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint8_t*)values_in,
+                         (const uint8_t*)nullptr, m, panels, (uint32_t)chunks, to_panel, (uint8_t*)values_out, (uint8_t*)nullptr);
+    return check_launch(fn);
+  }
   if (m <= 0 || m % 32 || k <= 0 || k % kp)
     return fail(TF24_ERR_SHAPE, "%s: shape (%lld, %lld): m must be a positive multiple of 32 and k of %lld", fn, (long long)m, (long long)k, (long long)kp);
+  // from here on the metadata moves through the word-by-word kernel: any pair with the reordered form, or metadata alone
   const bool panel_side = from_layout == TF24_COMPRESSED_PANEL || to_layout == TF24_COMPRESSED_PANEL;
-  if (!meta_in || !meta_out || (panel_side && (!values_in || !values_out))) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
+  if (!meta_in || !meta_out || (values_out && !values_in)) return fail(TF24_ERR_ARG, "%s: null pointer", fn);
   if (meta_in == meta_out || (values_out && values_in == values_out)) return fail(TF24_ERR_ARG, "%s: in-place conversion is not supported", fn);
   if ((values_out && ((uintptr_t)values_in | (uintptr_t)values_out) % 16) || ((uintptr_t)meta_in | (uintptr_t)meta_out) % 4)
     return fail(TF24_ERR_STRIDE, "%s: values must be 16-byte and metadata 4-byte aligned", fn);

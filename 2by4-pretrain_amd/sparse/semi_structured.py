@@ -58,12 +58,13 @@ def _panel_width(dtype):
     return 128 // torch.empty((), dtype=dtype).element_size()
 
 
-def _to_canonical(values, meta, m, n):
-    """Panel-layout storage -> canonical (values [m, n/2], meta [m, n/16 | n/32])."""
-    kp = _panel_width(values.dtype)
-    v = values.view(n // kp, m, kp // 2).permute(1, 0, 2).reshape(m, n // 2)
-    mt = meta.view(n // 32, m, 4 // meta.element_size()).permute(1, 0, 2).reshape(m, -1)   # [n/32][m][4 bytes] -> rows
-    return v, mt
+def _to_canonical(values, meta, m, n, want_values=True, want_meta=True):
+    """Panel-layout storage -> canonical (values [m, n/2], meta [m, n/16 | n/32]); None for a part not wanted."""
+    v = torch.empty_like(values) if want_values else None
+    mt = torch.empty_like(meta) if want_meta else None
+    N.check(N.lib().tf24_repack_to(values.data_ptr(), meta.data_ptr(), N.operand_code(values.dtype), m, n, N.COMPRESSED_PANEL,
+                                   N.COMPRESSED_CANONICAL, N.ptr(v), N.ptr(mt), N.stream_ptr()))
+    return (v.view(m, n // 2) if want_values else None), (mt.view(m, -1) if want_meta else None)
 
 
 class _HostWords:
@@ -367,35 +368,29 @@ class SparseSemiStructuredTensor(torch.Tensor):
         self._store_values, self._store_meta = values, meta       # flat device tensors
         self._store_shape, self._store_layout = shape, layout     # (m, k) of the untransposed matrix
 
-    def _canonical_pair(self):
+    def _canonical_pair(self, want_values=True, want_meta=True):
         """(values [m, k/2], canonical metadata) of the stored operand.  Made from the storage on every call
         (views where the storage is canonical, copies otherwise): the storage may be rewritten behind the
         wrapper's back -- a graph replay recompresses into the same buffers -- so nothing derived is kept."""
         m, n = self._store_shape
         if self._store_layout == N.COMPRESSED_PANEL:
-            return _to_canonical(self._store_values, self._store_meta, m, n)
+            return _to_canonical(self._store_values, self._store_meta, m, n, want_values, want_meta)
         if self._store_layout == N.COMPRESSED_CUTLASS:
-            return self._store_values.view(m, n // 2), self._converted_meta(N.COMPRESSED_CANONICAL)
+            return self._store_values.view(m, n // 2), (self._converted_meta(N.COMPRESSED_CANONICAL) if want_meta else None)
         return self._store_values.view(m, n // 2), self._store_meta.view(m, -1)
 
     def _converted_meta(self, to_layout):
         """The metadata in another storage form, [m, k/16 | k/32] words (HIP kernel; values untouched)."""
         m, n = self._store_shape
         out = torch.empty_like(self._store_meta)
-        if self._store_layout == N.COMPRESSED_PANEL:
-            # only the metadata is wanted: go through the canonical view of the panel words
-            src = self._canonical_pair()[1].contiguous()
-            N.check(N.lib().tf24_repack_to(None, src.data_ptr(), N.operand_code(self._store_values.dtype), m, n,
-                                           N.COMPRESSED_CANONICAL, to_layout, None, out.data_ptr(), N.stream_ptr()))
-        else:
-            N.check(N.lib().tf24_repack_to(None, self._store_meta.data_ptr(), N.operand_code(self._store_values.dtype), m, n,
-                                           self._store_layout, to_layout, None, out.data_ptr(), N.stream_ptr()))
+        N.check(N.lib().tf24_repack_to(None, self._store_meta.data_ptr(), N.operand_code(self._store_values.dtype), m, n,
+                                       self._store_layout, to_layout, None, out.data_ptr(), N.stream_ptr()))
         return out.view(m, -1)
 
     @property
     def sparse_tensor_cutlass(self):
         """Kept values, canonical [m, k/2] (the reference's attribute name)."""
-        return None if self._store_values is None else self._canonical_pair()[0]
+        return None if self._store_values is None else self._canonical_pair(want_meta=False)[0]
 
     @property
     def meta_tensor_cutlass(self):
@@ -403,7 +398,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
         `_CUTLASS_METADATA` the reference's reordered words."""
         if self._store_values is None:
             return None
-        return self.indices_cutlass() if self._CUTLASS_METADATA else self._canonical_pair()[1]
+        return self.indices_cutlass() if self._CUTLASS_METADATA else self._canonical_pair(want_values=False)[1]
 
     def __tensor_flatten__(self):
         return ["_store_values", "_store_meta"], (self.original_shape, self.transposed, self._store_shape, self._store_layout)
@@ -508,7 +503,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
 
     def indices_canonical(self):
         """Metadata as the canonical nibble stream, whatever `_CUTLASS_METADATA` says."""
-        return self._canonical_pair()[1]
+        return self._canonical_pair(want_values=False)[1]
 
     def indices_cutlass(self):
         """Metadata in the CUTLASS-reordered layout the reference's `indices()` returns

@@ -230,8 +230,8 @@ int tf24_repack(const void* values_in, const void* meta_in, int dtype, int64_t m
  * SparseSemiStructuredTensor.values() / indices() return (sparse/semi_structured.py:526-546); with to_layout
  * CUTLASS it is the reference's reordering step itself (sparse/_semi_structured_conversions.py:178-213,
  * Triton :639-661 and :1047-1069).  m % 32 == 0; k % 64 == 0 (16-bit values) / k % 128 == 0 (8-bit).
- * values_out may be NULL when neither side is PANEL (the values of CANONICAL and CUTLASS are the same bytes):
- * then only the metadata is converted.
+ * values_out NULL: only the metadata is converted (what indices() needs; the values of CANONICAL and CUTLASS are
+ * the same bytes anyway).  meta_out NULL, between CANONICAL and PANEL: only the values (what values() needs).
  */
 int tf24_repack_to(const void* values_in, const void* meta_in, int dtype, int64_t m, int64_t k, int from_layout,
                    int to_layout, void* values_out, void* meta_out, void* stream);
