@@ -285,3 +285,36 @@ def test_spmm_padded_leading_dimensions(cuda, dtype, n, k, j, sparse_first):
     rows, cols = want.shape
     assert wide_c[:, :cols].float().cpu().equal(want.float())
     assert bool((wide_c[:, cols:] == 7.0).all())
+
+
+@pytest.mark.parametrize("dtype,m,k", [(torch.float16, 352, 704), (torch.float8_e4m3fn, 96, 640)])
+def test_repack_to_one_part_only(cuda, dtype, m, k):
+    """tf24_repack_to with NULL for the part not wanted: values only between the canonical and the panel form,
+    metadata only between any two forms -- each equal to that part of the full conversion, the other output untouched."""
+    import sparse
+    N = sparse._native
+    w = _small_ints((m, k), 131).to(cuda)
+    s = sparse.to_sparse_semi_structured(w, dtype=dtype)
+    assert s._store_layout == N.COMPRESSED_PANEL
+    code = N.operand_code(dtype)
+    pv, pm = s._store_values, s._store_meta
+    cv, cm = torch.empty_like(pv), torch.empty_like(pm)
+    N.check(N.lib().tf24_repack_to(pv.data_ptr(), pm.data_ptr(), code, m, k, N.COMPRESSED_PANEL, N.COMPRESSED_CANONICAL, cv.data_ptr(), cm.data_ptr(), N.stream_ptr()))
+    bytes_of = lambda t: t.contiguous().view(torch.uint8)
+    for from_layout, to_layout, vin, min_, vwant, mwant in ((N.COMPRESSED_PANEL, N.COMPRESSED_CANONICAL, pv, pm, cv, cm),
+                                                           (N.COMPRESSED_CANONICAL, N.COMPRESSED_PANEL, cv, cm, pv, pm)):
+        v = torch.full_like(pv.view(torch.uint8), 0x5a)
+        N.check(N.lib().tf24_repack_to(vin.data_ptr(), None, code, m, k, from_layout, to_layout, v.data_ptr(), None, N.stream_ptr()))
+        assert v.equal(bytes_of(vwant).view_as(v))
+        mt = torch.full_like(pm.view(torch.uint8), 0x5a)
+        N.check(N.lib().tf24_repack_to(None, min_.data_ptr(), code, m, k, from_layout, to_layout, None, mt.data_ptr(), N.stream_ptr()))
+        assert mt.equal(bytes_of(mwant).view_as(mt))
+    # the reordered form: metadata straight from the panel words, and back
+    want = oracle.cutlass_reorder_meta(s.indices_canonical().cpu())
+    got = torch.empty_like(pm)
+    N.check(N.lib().tf24_repack_to(None, pm.data_ptr(), code, m, k, N.COMPRESSED_PANEL, N.COMPRESSED_CUTLASS, None, got.data_ptr(), N.stream_ptr()))
+    assert bytes_of(got).cpu().equal(bytes_of(want).view(-1).view_as(bytes_of(got).cpu()))
+    back = torch.empty_like(pm)
+    N.check(N.lib().tf24_repack_to(None, got.data_ptr(), code, m, k, N.COMPRESSED_CUTLASS, N.COMPRESSED_PANEL, None, back.data_ptr(), N.stream_ptr()))
+    assert bytes_of(back).equal(bytes_of(pm))
+    assert N.lib().tf24_repack_to(None, None, code, m, k, N.COMPRESSED_PANEL, N.COMPRESSED_CANONICAL, None, None, N.stream_ptr()) != 0
