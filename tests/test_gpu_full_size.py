@@ -214,3 +214,9 @@ def test_config5_fp8_spmm_rows_against_float32(cuda):
     sl = slice(16384 - 512, 16384)
     ref = torch.mm(aq[sl].float(), s.to_dense().float().t()) / (sa * sb)
     assert ((out[sl].float() - ref).norm() / ref.norm()).item() < 5e-2
+    # the reference's own output type for 8-bit operands is float32 (.cu:729, 772): the same accumulators through the
+    # 32-bit output pass, so rounding them to bf16 must give the bf16 product bit for bit, over all 2048 tiles
+    out32 = sparse.sparse_semi_structured_linear(aq, s, scale=1.0 / (sa * sb))
+    assert out32.dtype == torch.float32 and out32.shape == (16384, 8192)
+    assert torch.equal(out32.to(BF16), out)
+    assert ((out32[sl] - ref).norm() / ref.norm()).item() < 5e-2
