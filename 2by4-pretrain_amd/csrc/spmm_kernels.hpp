@@ -303,7 +303,7 @@ struct TileCfgT {
   static constexpr int TI = 4, TJ = TJ_;         // 32x32 instructions per wave
   static constexpr int WI = 32 * TI, WJ = 32 * TJ;
   static constexpr int BI = WI * WAVES_I, BJ = WJ * WAVES_J;
-  static_assert(BI == 256 && (BJ == 256 || BJ == 128 || BJ == 64), "stage buffers are sized for 256-row tiles of 256, 128 or 64 columns");
+  static_assert(BI == 256 && (BJ == 256 || BJ == 192 || BJ == 128 || BJ == 64), "stage buffers are sized for 256-row tiles of 256, 192, 128 or 64 columns");
   static constexpr int KB = 128;                 // bytes of dense k per row per stage
   static constexpr int STEPS = KB / 64;          // instruction steps per stage
   static constexpr int A_ROW = KB / 2;           // LDS bytes per row per stage: compressed values
@@ -323,6 +323,11 @@ using TiledCfg = TileCfgT<4, 2>;
 // 4-wave workgroup cost more than that (12 stages: 8 % slower; 24: equal; 32: 0.6 to 1.3 % faster), so only chained
 // tiles of kWave4MinStages or more stages take this form.
 using Wave4Cfg = TileCfgT<2, 4>;
+// 256 x 192 tiles in the 4-wave form (wave tile 128 x 96): a tile costs 0.89 of a 256 x 256 one, so where the
+// narrower tiles need no more rounds of the compute units than the wide ones, every round is that much shorter
+// (W[1600, 6400] against 12288 tokens: 336 wide tiles or 448 narrow ones, two rounds either way, 147 against 165 us;
+// W[11008, 4096] against 2048 tokens alike).  Long chained tiles only, like the 4-wave form itself.
+using Wave4Cfg192 = TileCfgT<2, 3>;
 constexpr int kWave4MinStages = 32;
 // 256 x 64 tiles, two waves: for dense operands of at most 64 columns (a few dozen tokens), where a
 // 256-wide tile would copy and multiply clamped columns.  26 KB per stage, two blocks per CU.
@@ -1000,10 +1005,23 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
                        k * (int64_t)sizeof(T) / C::KB >= 4 && per_xcd > cu_slots && cu_slots > 0;
   dim3 grid((unsigned)((persist ? cu_slots : per_xcd) * 8));
   const bool jm = c_layout == TF24_COL_MAJOR;
+  // long chained tiles of a k-contiguous dense operand take the 4-wave form
+  const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR &&
+                     k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages;
+  if constexpr (std::is_same<C, TiledCfg>::value && sizeof(OutT) == 2) {
+    const int tiles_j192 = (int)((n_dense + Wave4Cfg192::BJ - 1) / Wave4Cfg192::BJ);
+    const int per_xcd192 = (tiles_i * tiles_j192 + 7) / 8;
+    if (wave4 && per_xcd192 > cu_slots && (per_xcd192 + cu_slots - 1) / cu_slots <= (per_xcd + cu_slots - 1) / cu_slots) {
+      hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg192, false, true>), grid, dim3(Wave4Cfg192::THREADS), 0, s,
+                         (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                         (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace);
+      return check_launch("tf24_spmm");
+    }
+  }
   auto launch = [&](auto c_jmajor, auto b_kstrided) {
     if constexpr (C::BJ == 256 && decltype(c_jmajor)::value) {
       if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value) {
-        if (persist && k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages) {      // long chained tiles: the 4-wave form
+        if (wave4) {
           hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true>), grid, dim3(Wave4Cfg::THREADS), 0, s,
                              (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                              (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
