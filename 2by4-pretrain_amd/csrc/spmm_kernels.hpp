@@ -371,7 +371,7 @@ __global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
           OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act,
-          int tiles_i, int tiles_j, int splits, float* __restrict__ partial) {
+          int tiles_i, int tiles_j, int splits, float* __restrict__ partial, int stagger_ticks) {
   constexpr int ES = sizeof(T);
   constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
   constexpr int M_STEP = M_ROW / C::STEPS;
@@ -422,6 +422,17 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     tj0 = (int64_t)(in_group / gh) * C::BJ;
   };
   locate(unit, i0, j0);
+  // Chained tiles: every second workgroup of an XCD starts `stagger_ticks` (10 ns each) late.  All compute units
+  // otherwise finish their tiles at the same moment and write them out together, at the HBM rate, while no matrix
+  // instruction issues (a wave's stores share the counter its copies are waited on, so the next tile stalls until
+  // they are acknowledged); with two groups half a burst apart each group's stores drain while the other
+  // multiplies.  The wait is bounded by the clock itself.
+  if constexpr (PERSIST) {
+    if (stagger_ticks > 0 && ((bid >> 3) & 1)) {
+      const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
+      while (__builtin_amdgcn_s_memrealtime() - t0 < (uint64_t)stagger_ticks) __builtin_amdgcn_s_sleep(4);
+    }
+  }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1005,6 +1016,12 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
                        k * (int64_t)sizeof(T) / C::KB >= 4 && per_xcd > cu_slots && cu_slots > 0;
   dim3 grid((unsigned)((persist ? cu_slots : per_xcd) * 8));
   const bool jm = c_layout == TF24_COL_MAJOR;
+  // Start stagger of chained tiles (see spmm_pipe): half an output burst -- 256 tiles of 128 KB (16-bit) or 256 KB
+  // (32-bit) at the HBM write rate are 6 or 12 us -- where bursts recur or tiles are short.  Measured with 3 us on
+  // 16-bit outputs: 576 tiles of 12 stages 48.9 -> 43.4 us, 1376 tiles of 64 stages 0.361 -> 0.355 ms, 2048 tiles of
+  // 64 fp8 stages unchanged; 512 tiles of 172 stages (two rounds) lose 1 % and are left alone.
+  const int stagger_rounds = persist ? (per_xcd + cu_slots - 1) / cu_slots : 0;
+  const int stagger = (stagger_rounds >= 3 || (persist && k * (int64_t)sizeof(T) / C::KB <= 32)) ? (sizeof(OutT) == 2 ? 300 : 600) : 0;
   // long chained tiles of a k-contiguous dense operand take the 4-wave form
   const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR &&
                      k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages;
@@ -1014,7 +1031,7 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
     if (wave4 && per_xcd192 > cu_slots && (per_xcd192 + cu_slots - 1) / cu_slots <= (per_xcd + cu_slots - 1) / cu_slots) {
       hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg192, false, true>), grid, dim3(Wave4Cfg192::THREADS), 0, s,
                          (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
-                         (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace);
+                         (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace, stagger);
       return check_launch("tf24_spmm");
     }
   }
@@ -1024,20 +1041,20 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
         if (wave4) {
           hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true>), grid, dim3(Wave4Cfg::THREADS), 0, s,
                              (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
-                             (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
+                             (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace, stagger);
           return;
         }
       }
       if (persist) {
         hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, true>), grid, dim3(C::THREADS), 0, s,
                            (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
-                           (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
+                           (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace, stagger);
         return;
       }
     }
     hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, false>), grid, dim3(C::THREADS), 0, s,
                        (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
-                       (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace);
+                       (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace, 0);
   };
   bool kstrided = false;
   if constexpr (sizeof(T) == 2 && C::BJ == 256) kstrided = b_layout == TF24_COL_MAJOR;
