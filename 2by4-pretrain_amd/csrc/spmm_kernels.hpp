@@ -1017,11 +1017,14 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   dim3 grid((unsigned)((persist ? cu_slots : per_xcd) * 8));
   const bool jm = c_layout == TF24_COL_MAJOR;
   // Start stagger of chained tiles (see spmm_pipe): half an output burst -- 256 tiles of 128 KB (16-bit) or 256 KB
-  // (32-bit) at the HBM write rate are 6 or 12 us -- where bursts recur or tiles are short.  Measured with 3 us on
-  // 16-bit outputs: 576 tiles of 12 stages 48.9 -> 43.4 us, 1376 tiles of 64 stages 0.361 -> 0.355 ms, 2048 tiles of
-  // 64 fp8 stages unchanged; 512 tiles of 172 stages (two rounds) lose 1 % and are left alone.
+  // (32-bit) at the HBM write rate are 6 or 12 us -- for short tiles, whose time the bursts are a large part of, and
+  // for 32-bit outputs over three or more rounds.  Measured: 576 tiles of 12 stages 48.9 -> 43.4 us (the training
+  // step they belong to 0.684 -> 0.679 ms), 2048 tiles of 64 fp8 stages with float32 output 0.521 -> 0.514 ms; with
+  // 16-bit outputs the same tiles are unchanged and 1376 tiles of 64 fp16 stages lose 0.2 % (alternating with another
+  // product; 1.6 % faster when the same product repeats), so long 16-bit tiles start together.
   const int stagger_rounds = persist ? (per_xcd + cu_slots - 1) / cu_slots : 0;
-  const int stagger = (stagger_rounds >= 3 || (persist && k * (int64_t)sizeof(T) / C::KB <= 32)) ? (sizeof(OutT) == 2 ? 300 : 600) : 0;
+  const int stagger = !persist ? 0 : k * (int64_t)sizeof(T) / C::KB <= 32 ? (sizeof(OutT) == 2 ? 300 : 600)
+                               : (sizeof(OutT) == 4 && stagger_rounds >= 3) ? 600 : 0;
   // long chained tiles of a k-contiguous dense operand take the 4-wave form
   const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR &&
                      k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages;
