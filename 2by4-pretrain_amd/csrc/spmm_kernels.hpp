@@ -426,11 +426,12 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // otherwise finish their tiles at the same moment and write them out together, at the HBM rate, while no matrix
   // instruction issues (a wave's stores share the counter its copies are waited on, so the next tile stalls until
   // they are acknowledged); with two groups half a burst apart each group's stores drain while the other
-  // multiplies.  The wait is bounded by the clock itself.
+  // multiplies.
   if constexpr (PERSIST) {
     if (stagger_ticks > 0 && ((bid >> 3) & 1)) {
       const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
-      while (__builtin_amdgcn_s_memrealtime() - t0 < (uint64_t)stagger_ticks) __builtin_amdgcn_s_sleep(4);
+      for (int spin = 0; spin < 1024 && __builtin_amdgcn_s_memrealtime() - t0 < (uint64_t)stagger_ticks; spin++)
+        __builtin_amdgcn_s_sleep(4);                 // (also bounded in iterations, whatever the counter does)
     }
   }
 
