@@ -386,15 +386,20 @@ def train_workload(steps, warmup):
     ms/step of the sparse model and of the same MLP with dense nn.Linear layers, each issued eagerly and as
     replays of whole-step HIP graphs."""
     def timed(step_fn):
+        # median of three timed blocks of `steps` steps: the eager steps are issued by a Python thread whose
+        # pace moves by several per cent from one moment to the next on a shared host
         settle(lambda i: step_fn())
         for _ in range(warmup):
             step_fn()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            loss = step_fn()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / steps, loss.item()
+        blocks = []
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                loss = step_fn()
+            torch.cuda.synchronize()
+            blocks.append((time.perf_counter() - t0) * 1e3 / steps)
+        return sorted(blocks)[1], loss.item()
 
     out = {}
     for kind in ("sparse", "dense", "sparse_one_pass"):
@@ -414,6 +419,7 @@ def train_workload(steps, warmup):
 def train_record(r):
     """The training-step figures as they go into the JSON line."""
     return {
+        "timing": "every figure is the median of three consecutive timed blocks of `steps` steps",
         "ms_per_step": round(r["sparse_ms"], 4), "ms_per_step_with_MaskedDecayAdamW": round(r["sparse_one_pass_ms"], 4),
         "dense_autocast_ms_per_step": round(r["dense_ms"], 4),
         "speedup_vs_dense_step": round(r["dense_ms"] / r["sparse_ms"], 3),
