@@ -278,8 +278,9 @@ int tf24_adamw_masked_decay(float* p, const void* grad, int grad_dtype, float* e
 /*
  * The same update with the number of the update in device memory (int64, >= 1, advanced by the caller in
  * stream order before the call): the form a training step recorded into a HIP graph needs, where a host
- * number would be frozen at the recording -- what torch's optimizers call capturable.  The bias corrections
- * 1 - beta^step are formed on the device, in double like the host form's.
+ * number would be frozen at the recording -- what torch's optimizers call capturable; the reference's optimizer
+ * (sparse/adamw.py:83-84) keeps the count as a host integer only.  The bias corrections 1 - beta^step are formed on
+ * the device, in double like the host form's.
  */
 int tf24_adamw_masked_decay_device_step(float* p, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
                                         const void* mask, int mask_dtype, int64_t n, double lr, double beta1,
