@@ -215,10 +215,20 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
         if keep_panel:
             sparse._set_storage(pv, pm, (n, k), N.COMPRESSED_PANEL)
         values, meta, store_layout = pv, pm, N.COMPRESSED_PANEL
-    if dense.dtype != values.dtype:
-        raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {values.dtype}")
-    dense = N.as_matrix(dense)
-    lay, ld = N.layout_of(dense)
+    vdtype = values.dtype
+    if dense.dtype != vdtype:
+        raise RuntimeError(f"dense operand dtype {dense.dtype} does not match the sparse operand's {vdtype}")
+    # (layout, leading dimension) of the dense operand as it lies, or of a contiguous copy when the kernels cannot
+    # address it (N.as_matrix + N.layout_of, written out: this function is on the training step's host path)
+    d0, d1 = dense.shape
+    s0, s1 = dense.stride()
+    if s1 == 1 and s0 >= d1 and s0 % 8 == 0 and dense.data_ptr() % 16 == 0:
+        lay, ld = N.ROW_MAJOR, s0
+    elif s0 == 1 and s1 >= d0 and s1 % 8 == 0 and dense.data_ptr() % 16 == 0:
+        lay, ld = N.COL_MAJOR, s1
+    else:
+        dense = dense.contiguous()
+        lay, ld = N.ROW_MAJOR, dense.stride(0)
     # When k is the strided dimension of the dense operand (`S @ dense` with a row-major dense, e.g.
     # dW = MVUE(dY^T) @ x) the tiled kernel reads 16-bit operands as they are, transposing while it
     # loads fragments.  For 8-bit operands it wants k contiguous: one transposing copy of the dense
@@ -249,21 +259,26 @@ def _spmm(sparse, dense, sparse_first, bias=None, out_dtype=None, scale=1.0, act
     if kk != k:
         raise RuntimeError(f"inner dimensions do not match: sparse operand has k={k}, dense operand {tuple(dense.shape)}")
     if out_dtype is None:
-        out_dtype = torch.int32 if values.dtype == torch.int8 else torch.float32 if values.dtype in _FLOAT8 else values.dtype
-    out = torch.empty(out_shape, dtype=out_dtype, device=dense.device)
+        out_dtype = torch.int32 if vdtype == torch.int8 else torch.float32 if vdtype in _FLOAT8 else vdtype
+    device = dense.device
+    out = torch.empty(out_shape, dtype=out_dtype, device=device)
     if bias is not None:
-        bias = bias.to(out_dtype).contiguous()
+        if bias.dtype != out_dtype or not bias.is_contiguous():
+            bias = bias.to(out_dtype).contiguous()
         if bias.numel() != n:
             raise RuntimeError(f"bias must have {n} elements, got {bias.numel()}")
-    ws_key = (values.dtype, n, k, j)
+    code = N.operand_code(vdtype)
+    lib = N.lib()
+    ws_key = (vdtype, n, k, j)
     ws_bytes = _WORKSPACE_BYTES.get(ws_key)
     if ws_bytes is None:
-        ws_bytes = _WORKSPACE_BYTES[ws_key] = N.lib().tf24_spmm_workspace_bytes(N.operand_code(values.dtype), n, k, j)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dense.device) if ws_bytes else None
-    N.check(N.lib().tf24_spmm(
-        values.data_ptr(), meta.data_ptr(), store_layout, N.operand_code(values.dtype), n, k,
-        dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.operand_code(out_dtype), c_layout, out.stride(0),
-        N.ptr(bias), float(scale), activation, N.ptr(workspace), ws_bytes, N.stream_ptr()))
+        ws_bytes = _WORKSPACE_BYTES[ws_key] = lib.tf24_spmm_workspace_bytes(code, n, k, j)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    N.check(lib.tf24_spmm(
+        values.data_ptr(), meta.data_ptr(), store_layout, code, n, k,
+        dense.data_ptr(), b_layout, ld, j, out.data_ptr(), N.operand_code(out_dtype), c_layout, out_shape[1],
+        None if bias is None else bias.data_ptr(), float(scale), activation,
+        None if workspace is None else workspace.data_ptr(), ws_bytes, N.stream_ptr()))
     return out
 
 
@@ -271,9 +286,11 @@ def _dense_times_sparse_t(dense2d, sparse, bias=None):
     """dense2d @ S.t() (+ bias): what `torch.mm(x, S.t())` / `torch.addmm(bias, x, S.t())` dispatch to, without
     building the transposed wrapper and without the dispatcher round trip (some 40 us of host time per
     product, which a training step that is bound by its launch rate pays three times)."""
-    rows = dense2d.shape[0]
-    padded = sparse._pad_tensor_for_matmul(dense2d)
-    out = _spmm(sparse, padded, False, bias=bias, out_dtype=sparse._out_dtype())
+    rows, cols = dense2d.shape
+    cfg = _DTYPE_TO_SEMI_STRUCTURED_SPARSE_CONFIG[dense2d.dtype]
+    padded = dense2d if rows % cfg.dense_min_rows == 0 and cols % cfg.dense_min_cols == 0 else sparse._pad_tensor_for_matmul(dense2d)
+    out_dtype = sparse._FP8_OUT_DTYPE if sparse._store_values.dtype in _FLOAT8 else None
+    out = _spmm(sparse, padded, False, bias=bias, out_dtype=out_dtype)
     return out if padded is dense2d else out[:rows, :]
 
 
@@ -306,12 +323,7 @@ class SparseSemiStructuredTensor(torch.Tensor):
                 MVUE24: bool = False, mask: Optional[torch.Tensor] = None,
                 dtype: Optional[torch.dtype] = None, rand: Optional[torch.Tensor] = None):
         assert compressed_tensor_cusparselt is None or (sparse_tensor_cutlass is None and meta_tensor_cutlass is None)
-        if not cls._PROTOTYPE_WARNING_SHOWN:
-            warnings.warn(
-                "The PyTorch API of SparseSemiStructuredTensor is in prototype stage and will change in the "
-                "near future. Please open a Github issue for features requests and see our documentation on "
-                "the torch.sparse module for further information about the project.", UserWarning)
-            cls._PROTOTYPE_WARNING_SHOWN = True
+        cls._warn_once()
         if original_tensor is not None:
             previous, original_shape = original_tensor, original_tensor.shape
         elif compressed_tensor_cusparselt is not None:
@@ -412,11 +424,27 @@ class SparseSemiStructuredTensor(torch.Tensor):
             inner_tensors["_store_values"], inner_tensors["_store_meta"], store_shape, store_layout, original_shape, transposed)
 
     @classmethod
+    def _warn_once(cls):
+        if not cls._PROTOTYPE_WARNING_SHOWN:
+            warnings.warn(
+                "The PyTorch API of SparseSemiStructuredTensor is in prototype stage and will change in the "
+                "near future. Please open a Github issue for features requests and see our documentation on "
+                "the torch.sparse module for further information about the project.", UserWarning)
+            cls._PROTOTYPE_WARNING_SHOWN = True
+
+    @classmethod
     def _from_storage(cls, values, meta, store_shape, store_layout, shape, transposed):
-        m, n = store_shape
-        out = cls(None, original_shape=shape, sparse_tensor_cutlass=values.view(m, n // 2), meta_tensor_cutlass=meta,
-                  transposed=transposed, dtype=values.dtype)
-        out._set_storage(values, meta, store_shape, store_layout)
+        """A wrapper around storage that already exists (flat values and metadata in `store_layout`): what the
+        constructor builds from pieces, without its copies and checks -- the training layer makes six of these per step."""
+        cls._warn_once()
+        out = torch.Tensor._make_wrapper_subclass(cls, shape, device=values.device, dtype=values.dtype, layout=values.layout,
+                                                  requires_grad=False)
+        out._store_values, out._store_meta = values, meta
+        out._store_shape, out._store_layout = store_shape, store_layout
+        out.original_tensor = None
+        out.compressed_tensor_cusparselt = None
+        out.transposed = transposed
+        out.original_shape = shape
         return out
 
     def __repr__(self) -> str:  # type: ignore[override]
