@@ -121,27 +121,31 @@ __device__ __forceinline__ int finish_value(int accv, float, const OutT* bias, i
   return (act == TF24_ACT_RELU && v < 0) ? 0 : v;
 }
 
-// The output pass of the tiled kernel is compiled three times: without bias and activation, with a
-// bias only, and with both decided at run time.  Left to run-time tests alone, the per-element
-// selects and the inlined SiLU more than triple the time of the pass (21 000 against 6 300 cycles
-// per 256 x 256 tile), which is a tenth of the whole kernel at k = 4096.
-enum { EPI_PLAIN = 0, EPI_BIAS = 1, EPI_RUNTIME = 2, EPI_GELU = 3 };    // GELU: optional bias, then gelu_erf (the MLP's first layer)
-template <int MODE, typename OutT>
-__device__ __forceinline__ float finish_element(float accv, float scale, const OutT* bias, int64_t row, bool row_ok, int act) {
+// The output pass of the tiled kernel is compiled once per epilogue: plain, bias only, and bias (or none) followed by
+// each activation.  Left to run-time tests alone, the per-element selects and the inlined SiLU more than triple the
+// time of the pass (21 000 against 6 300 cycles per 256 x 256 tile), which is a tenth of the whole kernel at k = 4096.
+// The bias of an element arrives as a value: the pass reads it from LDS, where the wave has put the bias of its rows
+// (zeros without one).
+enum { EPI_PLAIN = 0, EPI_BIAS = 1, EPI_RELU = 2, EPI_SILU = 3, EPI_GELU = 4 };
+template <int MODE>
+__device__ __forceinline__ float finish_element(float accv, float scale, float biasv) {
   float v = accv * scale;
-  if constexpr (MODE == EPI_BIAS) { if (row_ok) v += to_float(bias[row]); }
-  if constexpr (MODE == EPI_RUNTIME) { if (bias && row_ok) v += to_float(bias[row]); v = apply_act(v, act); }
-  if constexpr (MODE == EPI_GELU) { if (bias && row_ok) v += to_float(bias[row]); v = gelu_erf(v); }
+  if constexpr (MODE != EPI_PLAIN) v += biasv;
+  if constexpr (MODE == EPI_RELU) v = v > 0.0f ? v : 0.0f;
+  if constexpr (MODE == EPI_SILU) v = v / (1.0f + __expf(-v));
+  if constexpr (MODE == EPI_GELU) v = gelu_erf(v);
   return v;
 }
-
-template <int MODE, typename OutT>
-__device__ __forceinline__ int finish_element(int accv, float, const OutT* bias, int64_t row, bool row_ok, int act) {
+// integer accumulators: bias and ReLU in int32, exact (the other activations are not defined for them)
+template <int MODE>
+__device__ __forceinline__ int finish_element(int accv, float, int biasv) {
   int v = accv;
-  if constexpr (MODE != EPI_PLAIN) { if (bias && row_ok) v += (int)bias[row]; }
-  if constexpr (MODE == EPI_RUNTIME) { if (act == TF24_ACT_RELU && v < 0) v = 0; }
+  if constexpr (MODE != EPI_PLAIN) v += biasv;
+  if constexpr (MODE == EPI_RELU) v = v < 0 ? 0 : v;
   return v;
 }
+template <typename OutT> __device__ __forceinline__ float bias_as(float, OutT b) { return to_float(b); }
+template <typename OutT> __device__ __forceinline__ int bias_as(int, OutT b) { return (int)b; }
 
 // ------------------------------------------------------------------------------------------
 // General kernel: operands straight from global memory (cached), every supported shape and
@@ -366,7 +370,10 @@ __device__ __forceinline__ void wait_reads_and_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <typename T, typename OutT, bool C_JMAJOR, typename C, bool B_KSTRIDED, bool PERSIST>
+// ACTS: the kernel is built twice, for launches without an activation (output pass: plain or bias only) and with one
+// (bias or zeros, then ReLU, SiLU or GELU); with all five passes in one kernel the compiler no longer keeps the
+// wave-uniform copy addresses in scalar registers.
+template <typename T, typename OutT, bool C_JMAJOR, typename C, bool B_KSTRIDED, bool PERSIST, bool ACTS = false>
 __global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
@@ -726,6 +733,22 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     else if (has_next) wait_reads_and_barrier();
     else stage_barrier(false);
   }
+  // ---- bias: every lane fetches the bias of WI/64 of its wave's rows here, one instruction step ahead of the
+  // output pass, which hands them round the wave through LDS.  (Fetched per element inside the pass -- 128 two-byte
+  // loads per lane, a wait behind every four -- the bias cost 2.8 us per 256 x 256 tile: 59 % on top of a 12-stage
+  // tile, 31 % on a 64-stage one.)
+  using accs_t = std::remove_reference_t<decltype(acc[0][0][0])>;
+  accs_t bias_v[C::WI / 64];
+#pragma unroll
+  for (int q = 0; q < C::WI / 64; q++) bias_v[q] = 0;
+  if (splits == 1 && bias != nullptr) {
+#pragma unroll
+    for (int q = 0; q < C::WI / 64; q++) {
+      const int64_t row = i0 + wi * C::WI + q * 64 + (int)(threadIdx.x & 63);
+      const accs_t v = bias_as(accs_t(0), bias[row < n_sparse ? row : n_sparse - 1]);
+      bias_v[q] = row < n_sparse ? v : accs_t(0);
+    }
+  }
   mma_step(1, 0, false, 0, 0, false, 0, 0);       // the last step
 
   // ---- split-K: park the 32-bit accumulators in the workspace, in register order (every group of
@@ -752,6 +775,18 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     int lane = threadIdx.x & 63;
     if constexpr (PERSIST) asm volatile("" : "+v"(lane));
     const int l32 = lane & 31, lh = lane >> 5;
+    // the bias of this wave's WI rows, behind the staging slices of all waves; the wave reads back what its own lanes
+    // wrote (LDS accesses of one wave execute in order: no barrier)
+    accs_t* bias_lds = reinterpret_cast<accs_t*>(smem + cur + C::NW * 4096 + wave * (C::WI * 4));
+    if constexpr (MODE != EPI_PLAIN) {
+#pragma unroll
+      for (int q = 0; q < C::WI / 64; q++) bias_lds[q * 64 + lane] = bias_v[q];
+    }
+    auto bias_quad = [&](int ti, int g) {            // the bias of rows ti*32 + g*8 + lh*4 + 0..3 of the wave's tile
+      typename mma32<T>::acc4_t q = {0, 0, 0, 0};
+      if constexpr (MODE != EPI_PLAIN) q = *reinterpret_cast<const typename mma32<T>::acc4_t*>(bias_lds + ti * 32 + g * 8 + lh * 4);
+      return q;
+    };
     // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
     // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
     // (8 bytes) in 32 different output rows, so direct stores would touch 32 lines per instruction.
@@ -774,12 +809,10 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             const int ti = ip * 2 + t2;
   #pragma unroll
             for (int g = 0; g < 4; g++) {
-              const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
               OutT o[4];
+              const auto bq = bias_quad(ti, g);
   #pragma unroll
-              for (int r = 0; r < 4; r++) {
-                o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
-              }
+              for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
               const int ch = t2 * 4 + g;
               *reinterpret_cast<Pack<OutT, 4>*>(stage + l32 * 128 + ((ch ^ (l32 & 7)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
             }
@@ -809,13 +842,11 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
         for (int ti = 0; ti < C::TI; ti++) {
   #pragma unroll
           for (int g = 0; g < 4; g++) {
-            const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
             typedef OutT out4v __attribute__((ext_vector_type(4)));
             out4v o;
+            const auto bq = bias_quad(ti, g);
   #pragma unroll
-            for (int r = 0; r < 4; r++) {
-              o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, row < n_sparse, act));
-            }
+            for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
             const int ch = g * 2 + lh;
             *reinterpret_cast<out4v*>(stage + l32 * 128 + ((ch ^ (l32 & 7)) * 16)) = o;
           }
@@ -846,14 +877,15 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             const int tj = half * 2 + t2;
             const int jl = t2 * 32 + l32;
   #pragma unroll
-            for (int g = 0; g < 4; g++)
+            for (int g = 0; g < 4; g++) {
+              const auto bq = bias_quad(ti, g);
   #pragma unroll
               for (int r = 0; r < 4; r++) {
                 const int il = g * 8 + lh * 4 + r;
-                const int64_t row = i0 + wi * C::WI + ti * 32 + il;
                 *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ (il & 7)) * 16) + (jl & 7) * 2) =
-                    to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row, row < n_sparse, act));
+                    to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
               }
+            }
           }
           const int64_t jcol = j0 + wj * C::WJ + half * 64 + chr * 8;
   #pragma unroll
@@ -876,10 +908,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
             if (col >= n_dense || row >= n_sparse) continue;
             OutT o[4];
+            const auto bq = bias_quad(ti, g);
   #pragma unroll
-            for (int r = 0; r < 4; r++) {
-              o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bias, row + r, true, act));
-            }
+            for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
             if constexpr (C_JMAJOR) {
               *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
             } else {
@@ -890,10 +921,18 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
         }
     }
   };
-  if (!bias && act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_PLAIN>{});
-  else if (act == TF24_ACT_NONE) output_pass(std::integral_constant<int, EPI_BIAS>{});
-  else if (act == TF24_ACT_GELU && !std::is_same<typename mma32<T>::acc4_t, int4v>::value) output_pass(std::integral_constant<int, EPI_GELU>{});
-  else output_pass(std::integral_constant<int, EPI_RUNTIME>{});
+  constexpr bool INT_ACC = std::is_same<typename mma32<T>::acc4_t, int4v>::value;
+  if constexpr (!ACTS) {
+    if (!bias) output_pass(std::integral_constant<int, EPI_PLAIN>{});
+    else output_pass(std::integral_constant<int, EPI_BIAS>{});
+  } else if constexpr (INT_ACC) {
+    if (act == TF24_ACT_RELU) output_pass(std::integral_constant<int, EPI_RELU>{});
+    else output_pass(std::integral_constant<int, EPI_BIAS>{});
+  } else {
+    if (act == TF24_ACT_RELU) output_pass(std::integral_constant<int, EPI_RELU>{});
+    else if (act == TF24_ACT_SILU) output_pass(std::integral_constant<int, EPI_SILU>{});
+    else output_pass(std::integral_constant<int, EPI_GELU>{});
+  }
   if (!has_next) break;
   // ---- the next tile: its first two stages are (about to be) in the buffers nxt and fre
   unit = next_unit; i0 = next_i0; j0 = next_j0; chained = true;
@@ -1027,7 +1066,8 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   const int stagger = !persist ? 0 : k * (int64_t)sizeof(T) / C::KB <= 32 ? (sizeof(OutT) == 2 ? 300 : 600)
                                : (sizeof(OutT) == 4 && stagger_rounds >= 3) ? 600 : 0;
   // long chained tiles of a k-contiguous dense operand take the 4-wave form
-  const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR &&
+  // (launches with an activation stay with the 8-wave form: one more pair of kernels to build otherwise)
+  const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR && act == TF24_ACT_NONE &&
                      k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages;
   if constexpr (std::is_same<C, TiledCfg>::value && sizeof(OutT) == 2) {
     const int tiles_j192 = (int)((n_dense + Wave4Cfg192::BJ - 1) / Wave4Cfg192::BJ);
@@ -1039,9 +1079,10 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
       return check_launch("tf24_spmm");
     }
   }
-  auto launch = [&](auto c_jmajor, auto b_kstrided) {
+  auto launch_epi = [&](auto c_jmajor, auto b_kstrided, auto acts) {
+    constexpr bool ACTS = decltype(acts)::value;
     if constexpr (C::BJ == 256 && decltype(c_jmajor)::value) {
-      if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value) {
+      if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value && !ACTS) {
         if (wave4) {
           hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true>), grid, dim3(Wave4Cfg::THREADS), 0, s,
                              (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
@@ -1050,15 +1091,20 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
         }
       }
       if (persist) {
-        hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, true>), grid, dim3(C::THREADS), 0, s,
+        hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, true, ACTS>), grid, dim3(C::THREADS), 0, s,
                            (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                            (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace, stagger);
         return;
       }
     }
-    hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, false>), grid, dim3(C::THREADS), 0, s,
+    hipLaunchKernelGGL((spmm_pipe<T, OutT, decltype(c_jmajor)::value, C, decltype(b_kstrided)::value, false, ACTS>), grid, dim3(C::THREADS), 0, s,
                        (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                        (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace, 0);
+  };
+  auto launch = [&](auto c_jmajor, auto b_kstrided) {
+    // with k pieces the reduction kernel applies bias and activation, not this one
+    if (act == TF24_ACT_NONE || splits > 1) launch_epi(c_jmajor, b_kstrided, std::false_type{});
+    else launch_epi(c_jmajor, b_kstrided, std::true_type{});
   };
   bool kstrided = false;
   if constexpr (sizeof(T) == 2 && C::BJ == 256) kstrided = b_layout == TF24_COL_MAJOR;

@@ -613,7 +613,8 @@ def test_spmm_chained_tiles_with_partial_edges(cuda, dtype, k):
                                                (F16, 320, "silu", 0.5), (BF16, 256, "gelu", 1.0), (E4M3, 640, "gelu", 0.125),
                                                (F16, 256, "gelu", 1.0), (E5M2, 512, "silu", 1.0)])
 def test_spmm_chained_tiles_activation_and_scale(cuda, dtype, k, act, scale):
-    """The chained-tile kernel's third output pass (bias, scale and activation decided at run time): 17 x 17
+    """The chained-tile kernel's output passes with an activation (the bias of a wave's rows reaches them through
+    LDS; zeros without a bias): 17 x 17
     tiles of 256 x 256 with partial edge tiles, more tiles than compute units.  Scale and bias act on exact
     float32 sums of small integers, so ReLU results are exact (one rounding of an exact value); SiLU and
     GELU are compared with torch's float32 functions of the same exact argument within 2e-3 + one unit in
@@ -639,6 +640,15 @@ def test_spmm_chained_tiles_activation_and_scale(cuda, dtype, k, act, scale):
         assert bool((err <= 2e-3 + (2e-3 + ulp) * want.abs()).all()), float(err.max())
     again = sparse.sparse_semi_structured_linear(x.to(cuda), s, bias_opt=bias.to(cuda), activation_opt=act, out_dtype=odt, scale=scale)
     assert again.equal(out)
+    # the same activation without a bias, right behind a launch that had one
+    nobias = sparse.sparse_semi_structured_linear(x.to(cuda), s, activation_opt=act, out_dtype=odt, scale=scale).float().cpu()
+    pre0 = pre - bias.float()
+    if act == "relu":
+        assert nobias.equal(pre0.clamp_min(0).to(odt).float())
+    else:
+        want0 = torch.nn.functional.silu(pre0) if act == "silu" else torch.nn.functional.gelu(pre0)
+        err0 = (nobias - want0).abs()
+        assert bool((err0 <= 2e-3 + (2e-3 + ulp) * want0.abs()).all()), float(err0.max())
 
 
 @pytest.mark.parametrize("dtype,k,act,n,m", [(F16, 1024, None, 4128, 4112), (BF16, 704, "relu", 4128, 4112),
