@@ -1072,7 +1072,12 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   if constexpr (std::is_same<C, TiledCfg>::value && sizeof(OutT) == 2) {
     const int tiles_j192 = (int)((n_dense + Wave4Cfg192::BJ - 1) / Wave4Cfg192::BJ);
     const int per_xcd192 = (tiles_i * tiles_j192 + 7) / 8;
-    if (wave4 && per_xcd192 > cu_slots && (per_xcd192 + cu_slots - 1) / cu_slots <= (per_xcd + cu_slots - 1) / cu_slots) {
+    // Also where both widths fit one round and the narrow tiles spread over more compute units (W[768, 3072] against
+    // 12288 tokens: 144 wide tiles or 192 narrow ones, 36.1 -> 34.1 us; W[1024, 4096]: 192 or 256 tiles, 56.2 -> 53.9 us).
+    const bool one_round192 = C::BJ == 256 && c_layout == TF24_COL_MAJOR && splits == 1 && b_layout == TF24_ROW_MAJOR && act == TF24_ACT_NONE &&
+                              k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages && cu_slots > 0 && per_xcd192 <= cu_slots && per_xcd192 > per_xcd;
+    if (one_round192 || (wave4 && per_xcd192 > cu_slots && (per_xcd192 + cu_slots - 1) / cu_slots <= (per_xcd + cu_slots - 1) / cu_slots)) {
+      if (one_round192) grid = dim3((unsigned)(cu_slots * 8));    // the chained-tile kernel with one tile per workgroup
       hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg192, false, true>), grid, dim3(Wave4Cfg192::THREADS), 0, s,
                          (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                          (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace, stagger);
