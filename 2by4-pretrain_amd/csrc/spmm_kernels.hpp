@@ -146,6 +146,17 @@ __device__ __forceinline__ int finish_element(int accv, float, int biasv) {
 }
 template <typename OutT> __device__ __forceinline__ float bias_as(float, OutT b) { return to_float(b); }
 template <typename OutT> __device__ __forceinline__ int bias_as(int, OutT b) { return (int)b; }
+// a bias element as the bits its load leaves in a register, and back
+template <typename OutT> __device__ __forceinline__ uint32_t bias_bits(OutT b) {
+  if constexpr (sizeof(OutT) == 2) { uint16_t h; __builtin_memcpy(&h, &b, 2); return h; }
+  else { uint32_t w; __builtin_memcpy(&w, &b, 4); return w; }
+}
+template <typename OutT> __device__ __forceinline__ OutT bias_from_bits(uint32_t w) {
+  OutT b;
+  if constexpr (sizeof(OutT) == 2) { const uint16_t h = (uint16_t)w; __builtin_memcpy(&b, &h, 2); }
+  else __builtin_memcpy(&b, &w, 4);
+  return b;
+}
 
 // ------------------------------------------------------------------------------------------
 // General kernel: operands straight from global memory (cached), every supported shape and
@@ -737,19 +748,24 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   // output pass, which hands them round the wave through LDS.  (Fetched per element inside the pass -- 128 two-byte
   // loads per lane, a wait behind every four -- the bias cost 2.8 us per 256 x 256 tile: 59 % on top of a 12-stage
   // tile, 31 % on a 64-stage one.)
+  // The loaded bits are first touched behind that step (the empty asm statements): converted right away, the compiler
+  // waits for each load -- and with it for every copy in flight -- before the step's matrix instructions.
   using accs_t = std::remove_reference_t<decltype(acc[0][0][0])>;
-  accs_t bias_v[C::WI / 64];
+  uint32_t bias_w[C::WI / 64];
 #pragma unroll
-  for (int q = 0; q < C::WI / 64; q++) bias_v[q] = 0;
+  for (int q = 0; q < C::WI / 64; q++) bias_w[q] = 0;
   if (splits == 1 && bias != nullptr) {
 #pragma unroll
     for (int q = 0; q < C::WI / 64; q++) {
       const int64_t row = i0 + wi * C::WI + q * 64 + (int)(threadIdx.x & 63);
-      const accs_t v = bias_as(accs_t(0), bias[row < n_sparse ? row : n_sparse - 1]);
-      bias_v[q] = row < n_sparse ? v : accs_t(0);
+      bias_w[q] = bias_bits(bias[row < n_sparse ? row : n_sparse - 1]);
     }
   }
   mma_step(1, 0, false, 0, 0, false, 0, 0);       // the last step
+  if (splits == 1 && bias != nullptr) {
+#pragma unroll
+    for (int q = 0; q < C::WI / 64; q++) asm volatile("" : "+v"(bias_w[q]));
+  }
 
   // ---- split-K: park the 32-bit accumulators in the workspace, in register order (every group of
   // four accumulators is one contiguous 16-byte-per-lane slab); spmm_reduce_splits finishes the job.
@@ -780,12 +796,21 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     accs_t* bias_lds = reinterpret_cast<accs_t*>(smem + cur + C::NW * 4096 + wave * (C::WI * 4));
     if constexpr (MODE != EPI_PLAIN) {
 #pragma unroll
-      for (int q = 0; q < C::WI / 64; q++) bias_lds[q * 64 + lane] = bias_v[q];
+      for (int q = 0; q < C::WI / 64; q++) {
+        const accs_t v = bias_as(accs_t(0), bias_from_bits<OutT>(bias_w[q]));
+        bias_lds[q * 64 + lane] = i0 + wi * C::WI + q * 64 + lane < n_sparse ? v : accs_t(0);
+      }
     }
-    auto bias_quad = [&](int ti, int g) {            // the bias of rows ti*32 + g*8 + lh*4 + 0..3 of the wave's tile
-      typename mma32<T>::acc4_t q = {0, 0, 0, 0};
-      if constexpr (MODE != EPI_PLAIN) q = *reinterpret_cast<const typename mma32<T>::acc4_t*>(bias_lds + ti * 32 + g * 8 + lh * 4);
-      return q;
+    // The bias of rows ti*32 + g*8 + lh*4 + 0..3 of the wave's tile, g = 0..3: read for a whole block of the pass
+    // ahead of its staging writes.  (Read where it is used, every quad waits behind the LDS writes issued before it,
+    // 32 round trips per wave and tile: 1.3 to 2 us.)
+    using bias4_t = typename mma32<T>::acc4_t;
+    auto bias_quads = [&](int ti, bias4_t (&bq)[4]) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        bq[g] = bias4_t{0, 0, 0, 0};
+        if constexpr (MODE != EPI_PLAIN) bq[g] = *reinterpret_cast<const bias4_t*>(bias_lds + ti * 32 + g * 8 + lh * 4);
+      }
     };
     // ---- epilogue.  D layout: column l%32, rows 8*(r/4) + 4*(l/32) + r%4.
     // For 16-bit outputs stored j-major (the Y of X.W^T) a lane owns runs of only 4 consecutive i
@@ -804,15 +829,17 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
       for (int tj = 0; tj < C::TJ; tj++) {
   #pragma unroll
         for (int ip = 0; ip < C::TI / 2; ip++) {                // 64 sparse rows (i) per pass
+          bias4_t bq[2][4];
+          bias_quads(ip * 2, bq[0]);
+          bias_quads(ip * 2 + 1, bq[1]);
   #pragma unroll
           for (int t2 = 0; t2 < 2; t2++) {
             const int ti = ip * 2 + t2;
   #pragma unroll
             for (int g = 0; g < 4; g++) {
               OutT o[4];
-              const auto bq = bias_quad(ti, g);
   #pragma unroll
-              for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
+              for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[t2][g][r]));
               const int ch = t2 * 4 + g;
               *reinterpret_cast<Pack<OutT, 4>*>(stage + l32 * 128 + ((ch ^ (l32 & 7)) * 16) + lh * 8) = *reinterpret_cast<Pack<OutT, 4>*>(o);
             }
@@ -840,13 +867,14 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
       for (int tj = 0; tj < C::TJ; tj++) {
   #pragma unroll
         for (int ti = 0; ti < C::TI; ti++) {
+          bias4_t bq[4];
+          bias_quads(ti, bq);
   #pragma unroll
           for (int g = 0; g < 4; g++) {
             typedef OutT out4v __attribute__((ext_vector_type(4)));
             out4v o;
-            const auto bq = bias_quad(ti, g);
   #pragma unroll
-            for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
+            for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[g][r]));
             const int ch = g * 2 + lh;
             *reinterpret_cast<out4v*>(stage + l32 * 128 + ((ch ^ (l32 & 7)) * 16)) = o;
           }
@@ -872,18 +900,19 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
       for (int half = 0; half < C::TJ / 2; half++) {            // 64 output columns (j) per pass
   #pragma unroll
         for (int ti = 0; ti < C::TI; ti++) {                    // 32 sparse rows (i) per pass
+          bias4_t bq[4];
+          bias_quads(ti, bq);
   #pragma unroll
           for (int t2 = 0; t2 < 2; t2++) {
             const int tj = half * 2 + t2;
             const int jl = t2 * 32 + l32;
   #pragma unroll
             for (int g = 0; g < 4; g++) {
-              const auto bq = bias_quad(ti, g);
   #pragma unroll
               for (int r = 0; r < 4; r++) {
                 const int il = g * 8 + lh * 4 + r;
                 *reinterpret_cast<OutT*>(stage + il * 128 + (((jl >> 3) ^ (il & 7)) * 16) + (jl & 7) * 2) =
-                    to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
+                    to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[g][r]));
               }
             }
           }
@@ -899,7 +928,9 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
       }
     } else {
   #pragma unroll
-      for (int ti = 0; ti < C::TI; ti++)
+      for (int ti = 0; ti < C::TI; ti++) {
+        bias4_t bq[4];
+        bias_quads(ti, bq);
   #pragma unroll
         for (int tj = 0; tj < C::TJ; tj++) {
           const int64_t col = j0 + wj * C::WJ + tj * 32 + l32;
@@ -908,9 +939,8 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             const int64_t row = i0 + wi * C::WI + ti * 32 + g * 8 + lh * 4;
             if (col >= n_dense || row >= n_sparse) continue;
             OutT o[4];
-            const auto bq = bias_quad(ti, g);
   #pragma unroll
-            for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[r]));
+            for (int r = 0; r < 4; r++) o[r] = to_out<OutT>(finish_element<MODE>(acc[ti][tj][g * 4 + r], scale, bq[g][r]));
             if constexpr (C_JMAJOR) {
               *reinterpret_cast<Pack<OutT, 4>*>(c + col * ldc + row) = *reinterpret_cast<Pack<OutT, 4>*>(o);
             } else {
@@ -919,6 +949,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
             }
           }
         }
+      }
     }
   };
   constexpr bool INT_ACC = std::is_same<typename mma32<T>::acc4_t, int4v>::value;
