@@ -389,7 +389,7 @@ __global__ void __launch_bounds__(C::THREADS)
 spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_meta, int64_t n_sparse, int64_t k,
           const uint8_t* __restrict__ b, int64_t ldb_bytes, int64_t n_dense,
           OutT* __restrict__ c, int64_t ldc, const OutT* __restrict__ bias, float scale, int act,
-          int tiles_i, int tiles_j, int splits, float* __restrict__ partial, int stagger_ticks) {
+          int tiles_i, int tiles_j, int splits, float* __restrict__ partial, int aux) {
   constexpr int ES = sizeof(T);
   constexpr int M_ROW = ES == 2 ? C::KB / 16 : C::KB / 8;   // metadata bytes per row per stage (8 or 16)
   constexpr int M_STEP = M_ROW / C::STEPS;
@@ -428,6 +428,10 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
   int unit = (bid & 7) * per_xcd + (bid >> 3);
   if (unit >= xcd_end) return;
   constexpr int GH = C::GH;
+  // aux: chained tiles (PERSIST) -- the start stagger in 10 ns ticks; otherwise the first row of tiles of this launch
+  // (a launch may cover the tile rows [aux, aux + tiles_i) of the product; n_sparse stays the row count of the whole operand)
+  const int stagger_ticks = PERSIST ? aux : 0;
+  const int tile_row0 = PERSIST ? 0 : aux;
   int split = 0;
   int64_t i0 = 0, j0 = 0;
   auto locate = [&](int u, int64_t& ti0, int64_t& tj0) {       // unit -> k piece and tile origin
@@ -436,7 +440,7 @@ spmm_pipe(const uint8_t* __restrict__ a_values, const uint8_t* __restrict__ a_me
     const int group = tile / (GH * tiles_j);
     const int gh = min(GH, tiles_i - group * GH);
     const int in_group = tile - group * GH * tiles_j;
-    ti0 = (int64_t)(group * GH + in_group % gh) * C::BI;
+    ti0 = (int64_t)(tile_row0 + group * GH + in_group % gh) * C::BI;
     tj0 = (int64_t)(in_group / gh) * C::BJ;
   };
   locate(unit, i0, j0);
@@ -1077,12 +1081,29 @@ template <typename T, typename OutT, typename C>
 int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, const void* b, int b_layout, int64_t ldb,
                  int64_t n_dense, void* c, int c_layout, int64_t ldc, const void* bias, float scale, int act,
                  void* workspace, int64_t workspace_bytes, hipStream_t s) {
-  const int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI), tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
+  int tiles_i = (int)((n_sparse + C::BI - 1) / C::BI);
+  const int tiles_j = (int)((n_dense + C::BJ - 1) / C::BJ);
   const int splits = workspace ? choose_splits<T, C>(n_sparse, k, n_dense, workspace_bytes) : 1;
+  const int cu_slots = compute_units() / 8;
+  // A last round that fills less than half of the compute units: the tile rows that make up the full rounds stay
+  // with the chained 256 x 256 tiles, the remaining rows go to a second launch on 256 x 128 tiles, which reach twice
+  // as many compute units for half the time each (W[11008, 4096] against 8192 tokens: 1376 tiles = 5 rounds of 256
+  // + 96; 40 tile rows chained, 3 rows as 192 half tiles: 351.6 -> 341.6 us).  Long tiles only: what a short
+  // tile's round costs is mostly its prologue and output pass, which the second launch pays again.
+  int tail_rows = 0;
+  if constexpr (std::is_same<C, TiledCfg>::value) {
+    const int cus = cu_slots * 8, tiles = tiles_i * tiles_j;
+    if (cus > 0 && c_layout == TF24_COL_MAJOR && b_layout == TF24_ROW_MAJOR && splits == 1 && tiles % cus != 0 &&
+        k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages) {
+      const int rows = tiles / cus * cus / tiles_j;            // tile rows of the full rounds
+      const int left = tiles_i - rows;
+      const int64_t half_tiles = (int64_t)left * ((n_dense + MidCfg::BJ - 1) / MidCfg::BJ);
+      if (rows * tiles_j > cus && left > 0 && half_tiles <= cus) { tiles_i = rows; tail_rows = left; }
+    }
+  }
   const int per_xcd = (tiles_i * tiles_j * splits + 7) / 8;
   // More tiles than compute units and no k pieces: one workgroup per compute unit walks its tiles in
   // one pipeline (the next tile's operands arrive while the current one is written out).
-  const int cu_slots = compute_units() / 8;
   const bool persist = C::BJ == 256 && c_layout == TF24_COL_MAJOR && splits == 1 &&
                        k * (int64_t)sizeof(T) / C::KB >= 4 && per_xcd > cu_slots && cu_slots > 0;
   dim3 grid((unsigned)((persist ? cu_slots : per_xcd) * 8));
@@ -1100,6 +1121,20 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   // (launches with an activation stay with the 8-wave form: one more pair of kernels to build otherwise)
   const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR && act == TF24_ACT_NONE &&
                      k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages;
+  auto launch_tail = [&]() {                       // the rows behind the full rounds, on 256 x 128 tiles
+    if constexpr (std::is_same<C, TiledCfg>::value) {
+      if (tail_rows > 0) {
+        const int tj = (int)((n_dense + MidCfg::BJ - 1) / MidCfg::BJ);
+        const dim3 tgrid((unsigned)((tail_rows * tj + 7) / 8 * 8));
+        auto tail = [&](auto acts) {
+          hipLaunchKernelGGL((spmm_pipe<T, OutT, true, MidCfg, false, false, decltype(acts)::value>), tgrid, dim3(MidCfg::THREADS), 0, s,
+                             (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                             (OutT*)c, ldc, (const OutT*)bias, scale, act, tail_rows, tj, 1, (float*)nullptr, tiles_i);
+        };
+        if (act == TF24_ACT_NONE) tail(std::false_type{}); else tail(std::true_type{});
+      }
+    }
+  };
   if constexpr (std::is_same<C, TiledCfg>::value && sizeof(OutT) == 2) {
     const int tiles_j192 = (int)((n_dense + Wave4Cfg192::BJ - 1) / Wave4Cfg192::BJ);
     const int per_xcd192 = (tiles_i * tiles_j192 + 7) / 8;
@@ -1112,6 +1147,7 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
       hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg192, false, true>), grid, dim3(Wave4Cfg192::THREADS), 0, s,
                          (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                          (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace, stagger);
+      launch_tail();
       return check_launch("tf24_spmm");
     }
   }
@@ -1153,6 +1189,7 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
     if (jm) launch(std::true_type{}, std::false_type{});
     else launch(std::false_type{}, std::false_type{});
   }
+  launch_tail();
   if (splits > 1) {
     dim3 rgrid((unsigned)(tiles_i * tiles_j), C::TI * C::TJ * 4);      // one accumulator group of the tile per block
     if (jm)

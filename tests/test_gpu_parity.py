@@ -658,12 +658,15 @@ def test_spmm_chained_tiles_activation_and_scale(cuda, dtype, k, act, scale):
                                               (E4M3, 6144, "relu", 4128, 4112), (E5M2, 6272, "silu", 4384, 4352),
                                               (F16, 2112, "relu", 1760, 12272), (E4M3, 4224, None, 1792, 12288),
                                               (BF16, 2048, "gelu", 2784, 8176), (F16, 2112, None, 800, 12272),
-                                              (BF16, 3072, None, 768, 12288)])
+                                              (BF16, 3072, None, 768, 12288), (F16, 2112, None, 4128, 8176),
+                                              (E4M3, 4224, "relu", 4128, 8176), (BF16, 2048, None, 4384, 8192)])
 def test_spmm_partial_last_round_long_k(cuda, dtype, k, act, n, m):
     """More tiles than compute units with a partial last round and 8 to 49 stages of k (the chained-tile kernel
     with one to three full rounds before the leftover tiles; from 32 stages on in its 4-wave form -- the last three
     shapes but two on 256 x 192 tiles, which need no more rounds there than 256 x 256 ones: 7 x 64 and 11 x 43 tiles with partial edges;
-    the last two on 4 x 64 and 3 x 64 such tiles in a single round, where 256 x 256 ones would leave compute units idle).  Sums of small integers are exact in float32, so the
+    the next two on 4 x 64 and 3 x 64 such tiles in a single round, where 256 x 256 ones would leave compute units idle;
+    the last three with two full rounds of 256 x 256 tiles and one or two more tile rows, which a second launch computes on
+    256 x 128 tiles -- in the first two of them the partial row of tiles).  Sums of small integers are exact in float32, so the
     results must equal the oracle's bit for bit, with bias, scale and activation behind the sum, for k contiguous
     and k strided dense operands, on a second call, and through the C ABI without a workspace."""
     import sparse
