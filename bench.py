@@ -867,7 +867,7 @@ def main():
     wall_ms, fwd_ms, bwd_ms, dfwd_ms, dbwd_ms, rel_f, rel_b, flops, (M, K, Nw) = spmm_workload(a.steps, a.warmup)
     value = 2 * flops / (wall_ms * 1e-3) / 1e12
     traffic_bytes, traffic_source = profiled_traffic()
-    dom_ms = (fwd_ms + bwd_ms) / 2                       # same kernel, two launches per step
+    dom_ms = (fwd_ms + bwd_ms) / 2                       # two products per step (the forward one: chained tiles + a launch for the last tile rows)
     executed_tflops = (flops / 2) / (dom_ms * 1e-3) / 1e12
     line = {
         "metric": "2:4 spMM TFLOP/s (dense-equivalent 2MNK; fwd X.W^T + transposed dY.W per step)",
@@ -881,9 +881,11 @@ def main():
                      "traffic": traffic_bytes,
                      "traffic_source": traffic_source,
                      "algorithmic_bytes": M * K * 2 + Nw * K * 9 // 8 + M * Nw * 2,
-                     "note": "achieved = executed flops (M*N*K, half the dense-equivalent 2MNK) per launch / HIP-event "
-                             "launch time; SMFMAC executes MACs at the dense MFMA rate, so frac also equals "
-                             "dense-equivalent rate / (2 x dense peak)",
+                     "note": "achieved = executed flops (M*N*K, half the dense-equivalent 2MNK) per product / HIP-event "
+                             "time of the product (one tf24_spmm call: the transposed product is one launch of the "
+                             "chained-tile kernel, the forward product that kernel on 1280 tiles + a launch on "
+                             "256 x 128 tiles for the last 3 tile rows); SMFMAC executes MACs at the dense MFMA rate, "
+                             "so frac also equals dense-equivalent rate / (2 x dense peak)",
                      "fwd_ms": round(fwd_ms, 4), "transposed_ms": round(bwd_ms, 4)},
         "dense_gemm": {"library": "torch.mm fp16 (hipBLASLt) on the masked dense weights",
                        "fwd_ms": round(dfwd_ms, 4), "transposed_ms": round(dbwd_ms, 4),
