@@ -1118,8 +1118,7 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   const int stagger = !persist ? 0 : k * (int64_t)sizeof(T) / C::KB <= 32 ? (sizeof(OutT) == 2 ? 300 : 600)
                                : (sizeof(OutT) == 4 && stagger_rounds >= 3) ? 600 : 0;
   // long chained tiles of a k-contiguous dense operand take the 4-wave form
-  // (launches with an activation stay with the 8-wave form: one more pair of kernels to build otherwise)
-  const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR && act == TF24_ACT_NONE &&
+  const bool wave4 = persist && std::is_same<C, TiledCfg>::value && b_layout == TF24_ROW_MAJOR &&
                      k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages;
   auto launch_tail = [&]() {                       // the rows behind the full rounds, on 256 x 128 tiles
     if constexpr (std::is_same<C, TiledCfg>::value) {
@@ -1140,13 +1139,16 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
     const int per_xcd192 = (tiles_i * tiles_j192 + 7) / 8;
     // Also where both widths fit one round and the narrow tiles spread over more compute units (W[768, 3072] against
     // 12288 tokens: 144 wide tiles or 192 narrow ones, 36.1 -> 34.1 us; W[1024, 4096]: 192 or 256 tiles, 56.2 -> 53.9 us).
-    const bool one_round192 = C::BJ == 256 && c_layout == TF24_COL_MAJOR && splits == 1 && b_layout == TF24_ROW_MAJOR && act == TF24_ACT_NONE &&
+    const bool one_round192 = C::BJ == 256 && c_layout == TF24_COL_MAJOR && splits == 1 && b_layout == TF24_ROW_MAJOR &&
                               k * (int64_t)sizeof(T) / C::KB >= kWave4MinStages && cu_slots > 0 && per_xcd192 <= cu_slots && per_xcd192 > per_xcd;
     if (one_round192 || (wave4 && per_xcd192 > cu_slots && (per_xcd192 + cu_slots - 1) / cu_slots <= (per_xcd + cu_slots - 1) / cu_slots)) {
       if (one_round192) grid = dim3((unsigned)(cu_slots * 8));    // the chained-tile kernel with one tile per workgroup
-      hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg192, false, true>), grid, dim3(Wave4Cfg192::THREADS), 0, s,
-                         (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
-                         (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace, stagger);
+      auto narrow = [&](auto acts) {
+        hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg192, false, true, decltype(acts)::value>), grid, dim3(Wave4Cfg192::THREADS), 0, s,
+                           (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
+                           (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j192, splits, (float*)workspace, stagger);
+      };
+      if (act == TF24_ACT_NONE) narrow(std::false_type{}); else narrow(std::true_type{});
       launch_tail();
       return check_launch("tf24_spmm");
     }
@@ -1154,9 +1156,9 @@ int launch_tiled(const void* av, const void* am, int64_t n_sparse, int64_t k, co
   auto launch_epi = [&](auto c_jmajor, auto b_kstrided, auto acts) {
     constexpr bool ACTS = decltype(acts)::value;
     if constexpr (C::BJ == 256 && decltype(c_jmajor)::value) {
-      if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value && !ACTS) {
+      if constexpr (std::is_same<C, TiledCfg>::value && !decltype(b_kstrided)::value) {
         if (wave4) {
-          hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true>), grid, dim3(Wave4Cfg::THREADS), 0, s,
+          hipLaunchKernelGGL((spmm_pipe<T, OutT, true, Wave4Cfg, false, true, ACTS>), grid, dim3(Wave4Cfg::THREADS), 0, s,
                              (const uint8_t*)av, (const uint8_t*)am, n_sparse, k, (const uint8_t*)b, ldb * (int64_t)sizeof(T), n_dense,
                              (OutT*)c, ldc, (const OutT*)bias, scale, act, tiles_i, tiles_j, splits, (float*)workspace, stagger);
           return;
